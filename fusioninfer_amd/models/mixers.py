@@ -28,6 +28,21 @@ model designs assemble them freely:
 * ``RoutedExperts``      mixture of gated feed-forward experts with a
   sigmoid or softmax router, top-k choice, optional renormalisation and a
   constant factor on the weights.
+* ``TemperedGatedAttention``  grouped-query softmax attention without
+  rotation: projection biases, a weighted RMS norm per query/key head, a
+  query factor that grows with the logarithm of the position's block
+  index, and a sigmoid gate per head on the result.
+* ``LatentAttention``    keys and values expanded from one normed low-rank
+  latent per token plus one rotated key part shared by all heads; only the
+  latent and the rotated part are cached, the expansions are folded into
+  the queries and the attended latents; optional per-head softmax sink.
+* ``RGLRUMixer``         real-gated linear recurrent unit behind a short
+  causal convolution with block-diagonal gates, times a GELU branch.
+* ``SquaredReluMLP``     down(relu(up x)^2) whose up projection may ride a
+  layer's merged input projection.
+* ``ParallelResidualLayer`` one layer norm feeding a mixer and a
+  feed-forward side by side, x <- x + m (mixer + ff), all input branches
+  in ONE merged projection.
 * ``GatedResidualLayer`` layer-normed residual layer whose sublayer
   results are multiplied by sigmoid(W h + b) before they are added; one
   mixer or several scaled mixers side by side behind ONE merged input
@@ -449,9 +464,10 @@ class GatedDeltaMixer(nn.Module):
 
 
 class RoutedExperts(nn.Module):
-    """Mixture of gated feed-forward experts: down(silu(gate x) * up x).
+    """Mixture of feed-forward experts: down(silu(gate x) * up x)
+    (``act`` "silu_gate") or down(relu(up x)^2) (``act`` "relu_sq").
 
-    Router logits are an fp32 product; scores are sigmoid(z) or
+    Router logits are an fp32 product (plus an optional bias); scores are sigmoid(z) or
     softmax(z); the ``top`` largest are chosen, optionally divided by their
     sum (+1e-20), and multiplied by ``scale``. On the GPU the experts run
     as two grouped GEMMs over block-aligned expert segments: the MFMA
@@ -460,10 +476,15 @@ class RoutedExperts(nn.Module):
 
     def __init__(self, width: int, ff: int, experts: int, top: int, dtype,
                  score: str = "sigmoid", renorm: bool = True,
-                 scale: float = 1.0):
+                 scale: float = 1.0, act: str = "silu_gate",
+                 router_bias: bool = False):
         super().__init__()
         if score not in ("sigmoid", "softmax"):
             raise ValueError(f"unknown router score {score!r}")
+        if act not in ("silu_gate", "relu_sq"):
+            raise ValueError(f"unknown expert activation {act!r}")
+        self.act = act
+        self.gated = act == "silu_gate"
         if not 1 <= top <= experts:
             raise ValueError("top must be in 1..experts")
         self.width, self.ff, self.experts, self.top = width, ff, experts, top
@@ -472,8 +493,12 @@ class RoutedExperts(nn.Module):
         self.router = nn.Parameter(
             torch.empty(experts, width, dtype=torch.float32).normal_(0, 0.02),
             requires_grad=False)
+        self.router_bias = (_f32_param((experts,), 0.0) if router_bias
+                            else None)
+        # gated: gate rows then up rows; otherwise the up rows alone
         self.gate_up = nn.Parameter(
-            torch.empty(experts, 2 * ff, width, dtype=dtype).normal_(0, 0.02),
+            torch.empty(experts, (2 if self.gated else 1) * ff, width,
+                        dtype=dtype).normal_(0, 0.02),
             requires_grad=False)
         self.down = nn.Parameter(
             torch.empty(experts, width, ff, dtype=dtype).normal_(0, 0.02),
@@ -512,7 +537,7 @@ class RoutedExperts(nn.Module):
     def route(self, x):
         from fusioninfer_amd import ops
 
-        logits = F.linear(x.float(), self.router)
+        logits = F.linear(x.float(), self.router, self.router_bias)
         return ops.moe_route(logits, self.top, self.score, self.renorm,
                              self.scale)
 
@@ -528,7 +553,11 @@ class RoutedExperts(nn.Module):
                 if rows.numel() == 0:
                     continue
                 gu = F.linear(x[rows], self.gate_up[e]).float()
-                act = (F.silu(gu[:, : self.ff]) * gu[:, self.ff:]).to(x.dtype)
+                if self.gated:
+                    act = (F.silu(gu[:, : self.ff])
+                           * gu[:, self.ff:]).to(x.dtype)
+                else:
+                    act = torch.relu(gu).pow(2).to(x.dtype)
                 y = F.linear(act, self.down[e]).float()
                 out.index_add_(0, rows, y * topv[rows, kk].unsqueeze(1))
             return out.to(x.dtype)
@@ -544,12 +573,14 @@ class RoutedExperts(nn.Module):
         if fast:
             gu_p, dn_p = self._packed_weights()
             ops.moe_gemm(act, x, gu_p, sorted_ids, expert_ids, n_valid,
-                         block_m, gate_up=True)
+                         block_m, gate_up=self.gated,
+                         up_act=None if self.gated else "relu_sq")
             ops.moe_gemm(y, act, dn_p, sorted_ids, expert_ids, n_valid,
                          block_m, gate_up=False)
         else:
             ops.moe_gemm_plain(act, x, self.gate_up, sorted_ids, expert_ids,
-                               n_valid, block_m, gate_up=True)
+                               n_valid, block_m, gate_up=self.gated,
+                               up_act=None if self.gated else "relu_sq")
             ops.moe_gemm_plain(y, act, self.down, sorted_ids, expert_ids,
                                n_valid, block_m, gate_up=False)
         out = torch.empty(T, self.width, dtype=x.dtype, device=x.device)
@@ -622,3 +653,291 @@ class GatedResidualLayer(nn.Module):
         return seqmix.gated_residual_layer_norm_(
             resid, self.mlp(h2), 1.0, None, 0.0, self.rg2(h2), self.rg2_bias,
             next_norm_w, self.eps, self.dtype)
+
+
+# ------------------------------------------------------------------------
+# Parallel-residual family of blocks
+
+
+@dataclasses.dataclass
+class TemperedGatedAttentionConfig:
+    heads: int
+    kv_heads: int
+    dim: int                 # per-head query/key size
+    vdim: int                # per-head value size
+    scale: float             # score multiplier
+    temp_coef: float = 0.0   # query factor 1 + coef * ln(floor((p+1)/every)+1)
+    temp_every: int = 0      # 0: no query temperature
+
+    def __post_init__(self):
+        if self.heads % self.kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+
+
+@dataclasses.dataclass
+class LatentAttentionConfig:
+    heads: int
+    dim: int                 # unrotated query/key size per head
+    rot_dim: int             # rotated query/key size (key part shared)
+    vdim: int
+    rank: int                # size of the cached latent
+    scale: float
+    rot_base: float
+    sink: bool = True        # learned per-head term in the denominator
+
+    def __post_init__(self):
+        if self.rot_dim % 2:
+            raise ValueError("rot_dim must be even")
+
+
+@dataclasses.dataclass
+class RGLRUConfig:
+    width: int               # channels of the recurrence
+    blocks: int              # block-diagonal gate matrices
+    conv: int                # taps of the causal convolution
+    # log a = -decay_scale * r * softplus(lam): the unit's fixed constant
+    decay_scale: float = 8.0
+
+    def __post_init__(self):
+        if self.width % self.blocks:
+            raise ValueError("width must be a multiple of blocks")
+        if self.conv < 1:
+            raise ValueError("conv taps must be >= 1")
+
+
+class TemperedGatedAttention(nn.Module):
+    """q, k, v and the per-head gate come from the merged projection (the
+    gate's rows carry a zero bias)."""
+
+    has_bias = True
+    biased = ("q", "k", "v")
+
+    def __init__(self, cfg: TemperedGatedAttentionConfig, width: int,
+                 eps: float, dtype):
+        super().__init__()
+        self.cfg = cfg
+        self.eps = eps
+        self.dtype = dtype
+        self.in_sizes = [cfg.heads * cfg.dim, cfg.kv_heads * cfg.dim,
+                         cfg.kv_heads * cfg.vdim, cfg.heads]
+        self.in_names = ["q", "k", "v", "g"]
+        self.q_norm = _f32_param((cfg.dim,), 1.0)
+        self.k_norm = _f32_param((cfg.dim,), 1.0)
+        self.o_proj = RowParallelLinear(cfg.heads * cfg.vdim, width,
+                                        dtype=dtype)
+
+    def state_tensors(self, num_blocks, block_size, num_slots, device):
+        c = self.cfg
+        return {
+            "k": torch.zeros((num_blocks, c.kv_heads, block_size, c.dim),
+                             dtype=self.dtype, device=device),
+            "v": torch.zeros((num_blocks, c.kv_heads, block_size, c.vdim),
+                             dtype=self.dtype, device=device),
+        }
+
+    def block_bytes(self, block_size: int) -> int:
+        c = self.cfg
+        esize = torch.empty((), dtype=self.dtype).element_size()
+        return c.kv_heads * block_size * (c.dim + c.vdim) * esize
+
+    def forward(self, parts, meta, cache) -> torch.Tensor:
+        q, k, v, g = parts
+        c = self.cfg
+        qn = seqmix.headnorm_qtemp_cache_(
+            q, k, v, meta.positions, self.q_norm, self.k_norm, self.eps,
+            c.temp_coef, c.temp_every, cache["k"], cache["v"],
+            meta.slot_mapping, c.heads, c.kv_heads, c.dim, c.vdim)
+        o = seqmix.sink_paged_attention(
+            qn, cache["k"], cache["v"], meta.seq_bt, meta.row_seq,
+            meta.positions, c.scale, out_gate=g, seq_cu=meta.seq_cu,
+            tiles=meta.seq_tiles)
+        return self.o_proj(o.view(o.shape[0], c.heads * c.vdim))
+
+
+class LatentAttention(nn.Module):
+    """q and the down projection (latent | shared rotated key part) come
+    from the merged projection. The key expansion is folded into the
+    queries (q_h^T W_uk,h) and the value expansion applied to the attended
+    latents, so attention runs over the cached rows [latent | rotated
+    part] with one shared key/value head."""
+
+    has_bias = False
+
+    def __init__(self, cfg: LatentAttentionConfig, width: int, eps: float,
+                 dtype):
+        super().__init__()
+        self.cfg = cfg
+        self.eps = eps
+        self.dtype = dtype
+        H = cfg.heads
+        self.in_sizes = [H * (cfg.dim + cfg.rot_dim), cfg.rank + cfg.rot_dim]
+        self.in_names = ["q", "dkv"]
+        self.c_norm = _f32_param((cfg.rank,), 1.0)
+        self.uk = nn.Parameter(
+            torch.empty(H * cfg.dim, cfg.rank, dtype=dtype).normal_(0, 0.02),
+            requires_grad=False)
+        self.uv = nn.Parameter(
+            torch.empty(H * cfg.vdim, cfg.rank, dtype=dtype).normal_(0, 0.02),
+            requires_grad=False)
+        self.sink = _f32_param((H,), 0.0) if cfg.sink else None
+        self.o_proj = RowParallelLinear(H * cfg.vdim, width, dtype=dtype)
+        self.register_buffer(
+            "inv_freq", rotary_inv_freq(cfg.rot_dim, cfg.rot_base),
+            persistent=False)
+
+    def state_tensors(self, num_blocks, block_size, num_slots, device):
+        c = self.cfg
+        return {"kv": torch.zeros(
+            (num_blocks, 1, block_size, c.rank + c.rot_dim),
+            dtype=self.dtype, device=device)}
+
+    def block_bytes(self, block_size: int) -> int:
+        c = self.cfg
+        esize = torch.empty((), dtype=self.dtype).element_size()
+        return block_size * (c.rank + c.rot_dim) * esize
+
+    def forward(self, parts, meta, cache) -> torch.Tensor:
+        q, dkv = parts
+        c = self.cfg
+        T, H = q.shape[0], c.heads
+        qf = torch.empty((T, H, c.rank + c.rot_dim), dtype=q.dtype,
+                         device=q.device)
+        seqmix.latent_rope_cache_(
+            q, dkv, meta.positions, self.inv_freq, self.c_norm, self.eps,
+            cache["kv"], meta.slot_mapping, H, c.dim, c.rot_dim, c.rank, qf)
+        # fold the key expansion into the queries: [H, T, dim] x [H, dim, rank]
+        qu = q.view(T, H, c.dim + c.rot_dim)[:, :, : c.dim].transpose(0, 1)
+        qf[:, :, : c.rank] = torch.bmm(
+            qu, self.uk.view(H, c.dim, c.rank)).transpose(0, 1)
+        o = seqmix.sink_paged_attention(
+            qf, cache["kv"], None, meta.seq_bt, meta.row_seq, meta.positions,
+            c.scale, sink=self.sink, value_dims=c.rank, seq_cu=meta.seq_cu,
+            tiles=meta.seq_tiles)
+        # expand the attended latents: [H, T, rank] x [H, rank, vdim]
+        ov = torch.bmm(o.transpose(0, 1),
+                       self.uv.view(H, c.vdim, c.rank).transpose(1, 2))
+        return self.o_proj(ov.transpose(0, 1).reshape(T, H * c.vdim))
+
+
+class RGLRUMixer(nn.Module):
+    """Recurrent block: the GELU branch and the convolved branch come from
+    the merged projection (both with biases). The block-diagonal gate
+    products run in fp32 as one batched GEMM."""
+
+    has_bias = True
+    biased = ("y", "x")
+
+    def __init__(self, cfg: RGLRUConfig, width: int, eps: float, dtype):
+        super().__init__()
+        self.cfg = cfg
+        self.dtype = dtype
+        W, B = cfg.width, cfg.blocks
+        bw = W // B
+        self.in_sizes = [W, W]
+        self.in_names = ["y", "x"]
+        conv = torch.zeros(W, cfg.conv, dtype=torch.float32)
+        conv[:, -1] = 1.0
+        self.conv_w = nn.Parameter(conv, requires_grad=False)
+        self.conv_b = _f32_param((W,), 0.0)
+        # per block: recurrence-gate rows then input-gate rows, [out, in]
+        self.gate_w = nn.Parameter(
+            torch.empty(B, 2 * bw, bw, dtype=torch.float32).normal_(
+                0, 1.0 / math.sqrt(bw)), requires_grad=False)
+        self.gate_b = _f32_param((B, 2 * bw), 0.0)
+        self.lam = _f32_param((W,), 0.0)
+        self.o_proj = RowParallelLinear(W, width, dtype=dtype)
+
+    def state_tensors(self, num_blocks, block_size, num_slots, device):
+        c = self.cfg
+        return {
+            "conv": torch.zeros((num_slots, max(c.conv - 1, 1), c.width),
+                                dtype=torch.float32, device=device),
+            "lru": torch.zeros((num_slots, c.width), dtype=torch.float32,
+                               device=device),
+        }
+
+    def block_bytes(self, block_size: int) -> int:
+        return 0
+
+    def forward(self, parts, meta, cache) -> torch.Tensor:
+        y_lin, x_lin = parts
+        c = self.cfg
+        T, B = y_lin.shape[0], c.blocks
+        u = seqmix.causal_conv_state(
+            x_lin, self.conv_w, self.conv_b, cache["conv"], meta.seq_cu,
+            meta.row_seq, meta.seq_slots, meta.positions)
+        gates = torch.bmm(u.view(T, B, c.width // B).transpose(0, 1),
+                          self.gate_w.transpose(1, 2))
+        o = seqmix.rglru_scan(
+            u, gates, self.gate_b, self.lam, y_lin, cache["lru"],
+            meta.seq_cu, meta.seq_slots, meta.positions, c.decay_scale,
+            self.dtype, max_rows=meta.max_seq_rows)
+        return self.o_proj(o)
+
+
+class SquaredReluMLP(nn.Module):
+    """down(relu(up x)^2). With ``own_up`` False the up projection is a
+    branch of the caller's merged projection and forward takes its
+    result."""
+
+    def __init__(self, width: int, ff: int, dtype, own_up: bool = True):
+        super().__init__()
+        self.ff = ff
+        self.up_proj = (ReplicatedLinear(width, ff, dtype=dtype)
+                        if own_up else None)
+        self.down_proj = RowParallelLinear(ff, width, dtype=dtype)
+
+    def forward(self, x):
+        if self.up_proj is not None:
+            x = self.up_proj(x)
+        return self.down_proj(seqmix.relu_squared(x))
+
+
+class ParallelResidualLayer(nn.Module):
+    """x <- x + mult * (mixer(h) + ff(h)),  h = layer_norm(x) w,
+    with the residual stream x kept in fp32. The mixer's input branches
+    and the up projection of the dense feed-forward (or of the shared
+    expert) are one merged projection of h; routed experts read h
+    themselves. ``forward`` receives h and returns the next layer's normed
+    input (None when ``next_norm_w`` is None), so the residual update is
+    fused with the norm that follows it."""
+
+    def __init__(self, mixer: nn.Module, dense: Optional[SquaredReluMLP],
+                 routed: Optional[nn.Module], width: int, eps: float,
+                 mult: float, dtype):
+        super().__init__()
+        self.mixer = mixer
+        self.dense = dense          # dense feed-forward or shared expert
+        self.routed = routed
+        self.eps = eps
+        self.mult = float(mult)
+        self.dtype = dtype
+        self.width = width
+        self.branches: List[str] = list(mixer.in_names)
+        self.sizes: List[int] = list(mixer.in_sizes)
+        if dense is not None:
+            self.branches.append("up")
+            self.sizes.append(dense.ff)
+        self.in_proj = MergedColumnParallelLinear(
+            width, self.sizes, dtype=dtype, bias=mixer.has_bias)
+        self.norm1 = _f32_param((width,), 1.0)
+
+    def in_proj_rows(self, branch: str):
+        off = 0
+        for name, size in zip(self.branches, self.sizes):
+            if name == branch:
+                return off, size
+            off += size
+        raise KeyError(branch)
+
+    def forward(self, resid, h, meta, cache, next_norm_w):
+        parts = self.in_proj(h).split(self.sizes, dim=-1)
+        n = len(self.mixer.in_sizes)
+        ys = [self.mixer(parts[:n], meta, cache)]
+        if self.dense is not None:
+            ys.append(self.dense(parts[n]))
+        if self.routed is not None:
+            ys.append(self.routed(h))
+        return seqmix.scaled_residual_layer_norm_(
+            resid, ys, [self.mult] * len(ys), next_norm_w, self.eps,
+            self.dtype)

@@ -254,6 +254,19 @@ def _register_builtin_architectures() -> None:
     register_architecture("Sefalorn", sefalorn_config, sefalorn_model,
                           extensions=("seqmix", "moe"))
 
+    def momedra_config(raw, model_path):
+        from fusioninfer_amd.models import momedra
+
+        return momedra.model_config_from_dict(raw, model_path)
+
+    def momedra_model(cfg):
+        from fusioninfer_amd.models.momedra import MomedraLM
+
+        return MomedraLM(cfg)
+
+    register_architecture("Momedra", momedra_config, momedra_model,
+                          extensions=("seqmix", "moe"))
+
 
 _register_builtin_architectures()
 

@@ -386,31 +386,45 @@ def has_moe_native() -> bool:
         return False
 
 
+def _moe_gemm_mode(gate_up: bool, up_act) -> int:
+    """0: plain GEMM over act rows; 1: gathered x rows, gate|up columns,
+    silu(gate) * up; 2: gathered x rows, up columns alone, relu(up)^2."""
+    if up_act is None:
+        return 1 if gate_up else 0
+    if up_act != "relu_sq" or gate_up:
+        raise ValueError(f"unsupported expert activation {up_act!r}")
+    return 2
+
+
 def moe_gemm(out, a, b_packed, sorted_ids, expert_ids, n_valid,
-             block_m: int, gate_up: bool):
+             block_m: int, gate_up: bool, up_act=None):
     """Grouped GEMM over block-aligned expert segments.
 
     out [PM, N] bf16; a = x [T, K] (gate_up, rows gathered via sorted_ids)
     or act [PM, K]; b_packed from pack_moe_weights ([E, K/32, NB/16, 64, 8]
     with NB = 2N when gate_up). n_valid: device int32 scalar tensor with
     the real m-tile count (static grid, dynamic work — hipGraph-safe).
-    gate_up=True fuses the SwiGLU epilogue: out = silu(gate) * up."""
+    gate_up=True fuses the SwiGLU epilogue: out = silu(gate) * up.
+    up_act="relu_sq" (with gate_up=False): a = x gathered like gate_up,
+    b holds the up matrix alone and out = relu(a @ up)^2."""
+    mode = _moe_gemm_mode(gate_up, up_act)
     if out.is_cuda:
         _moe_native().moe_gemm(out, a, b_packed, sorted_ids, expert_ids,
-                               n_valid, block_m, gate_up)
+                               n_valid, block_m, mode)
         return out
     return ref.moe_gemm(out, a, b_packed, sorted_ids, expert_ids, n_valid,
-                        block_m, gate_up)
+                        block_m, gate_up, up_act)
 
 
 def moe_gemm_plain(out, a, w, sorted_ids, expert_ids, n_valid, block_m: int,
-                   gate_up: bool):
+                   gate_up: bool, up_act=None):
     """Grouped GEMM of the same block-aligned layout for ANY sizes and for
     fp32 or bf16 operands (fp32 accumulation): w is the experts' natural
     [E, out, in] weight ([E, 2N, K] with gate rows first when gate_up,
-    which also applies out = silu(gate) * up). GPU only."""
+    which also applies out = silu(gate) * up; up_act="relu_sq": [E, N, K]
+    up rows alone on gathered x rows, out = relu(.)^2). GPU only."""
     _moe_native().moe_gemm_plain(out, a, w, sorted_ids, expert_ids, n_valid,
-                                 block_m, gate_up)
+                                 block_m, _moe_gemm_mode(gate_up, up_act))
     return out
 
 

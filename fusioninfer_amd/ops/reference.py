@@ -313,7 +313,7 @@ def unpack_moe_weights(b_packed: torch.Tensor) -> torch.Tensor:
 
 
 def moe_gemm(out, a, b_packed, sorted_ids, expert_ids, n_valid,
-             block_m: int, gate_up: bool):
+             block_m: int, gate_up: bool, up_act=None):
     """fp32 reference of the grouped GEMM (CPU; same semantics as the HIP
     kernel incl. padding rows computed from the dummy token row)."""
     w = unpack_moe_weights(b_packed).float()
@@ -323,7 +323,7 @@ def moe_gemm(out, a, b_packed, sorted_ids, expert_ids, n_valid,
         e = int(expert_ids[mt])
         r0 = mt * block_m
         rows = slice(r0, r0 + block_m)
-        if gate_up:
+        if gate_up or up_act is not None:
             src = a[sorted_ids[rows].long()].float()
         else:
             src = a[rows].float()
@@ -331,6 +331,8 @@ def moe_gemm(out, a, b_packed, sorted_ids, expert_ids, n_valid,
         if gate_up:
             g, u = acc[:, :N], acc[:, N:]
             acc = torch.nn.functional.silu(g) * u
+        elif up_act == "relu_sq":
+            acc = torch.relu(acc).pow(2)
         out[rows] = acc.to(out.dtype)
     return out
 

@@ -339,3 +339,139 @@ def gated_delta_rule(x, conv_w, alin, blin, a_log, dt_bias, conv_state,
     return ref.gated_delta_rule(x, conv_w, alin, blin, a_log, dt_bias,
                                 conv_state, state, seq_cu, seq_slots,
                                 positions, heads, kv_heads, dim, vdim)
+
+
+# ------------------------------------------------------------------------
+# parallel-residual stream, weighted head norms with a query temperature,
+# latent keys/values with a softmax sink, gated linear recurrence
+
+def scaled_residual_layer_norm_(resid, ys, scales, w_next, eps: float,
+                                out_dtype):
+    """resid (fp32, in place) += sum_i scales[i] * ys[i] for one to three
+    sublayer results; returns layer_norm(resid) * w_next (None without
+    w_next)."""
+    if not 1 <= len(ys) <= 3 or len(ys) != len(scales):
+        raise ValueError("one to three terms, one scale each")
+    if resid.is_cuda:
+        out = None
+        if w_next is not None:
+            out = torch.empty(resid.shape, dtype=out_dtype,
+                              device=resid.device)
+        ys = list(ys) + [None] * (3 - len(ys))
+        sc = [float(s) for s in scales] + [0.0] * (3 - len(scales))
+        _native().scaled_residual_layer_norm(resid, ys[0], sc[0], ys[1],
+                                             sc[1], ys[2], sc[2], w_next,
+                                             out, eps)
+        return out
+    return ref.scaled_residual_layer_norm_(resid, ys, scales, w_next, eps,
+                                           out_dtype)
+
+
+def headnorm_qtemp_cache_(q, k, v, positions, q_w, k_w, eps: float,
+                          temp_coef: float, temp_every: int, k_cache,
+                          v_cache, slot_mapping, num_heads: int,
+                          num_kv_heads: int, dim: int, vdim: int):
+    """q/k/v may be column slices of one projection output; returns a
+    fresh contiguous processed q [T, H, dim]."""
+    if q.is_cuda:
+        out = torch.empty((q.shape[0], num_heads, dim), dtype=q.dtype,
+                          device=q.device)
+        _native().headnorm_qtemp_cache(out, q, k, v, positions, q_w, k_w,
+                                       eps, float(temp_coef),
+                                       int(temp_every), k_cache, v_cache,
+                                       slot_mapping, num_heads,
+                                       num_kv_heads, dim, vdim)
+        return out
+    return ref.headnorm_qtemp_cache_(q, k, v, positions, q_w, k_w, eps,
+                                     temp_coef, temp_every, k_cache, v_cache,
+                                     slot_mapping, num_heads, num_kv_heads,
+                                     dim, vdim)
+
+
+def latent_rope_cache_(q, ckr, positions, inv_freq, norm_w, eps: float,
+                       kv_cache, slot_mapping, num_heads: int, dim: int,
+                       rot_dim: int, rank: int, q_out):
+    """Writes the rotated query parts into q_out[:, :, rank:] ([T, H,
+    rank+rot_dim]) and the normed latent + rotated shared key part into
+    the paged cache."""
+    if q.is_cuda:
+        _native().latent_rope_cache(q_out, q, ckr, positions, inv_freq,
+                                    norm_w, eps, kv_cache, slot_mapping,
+                                    num_heads, dim, rot_dim, rank)
+        return
+    ref.latent_rope_cache_(q, ckr, positions, inv_freq, norm_w, eps,
+                           kv_cache, slot_mapping, num_heads, dim, rot_dim,
+                           rank, q_out)
+
+
+def sink_paged_attention(q, k_cache, v_cache, seq_bt, row_seq, positions,
+                         scale: float, sink=None, value_dims: int = 0,
+                         out_gate=None, seq_cu=None, tiles=None):
+    """Causal softmax attention over the paged cache with separate key and
+    value sizes, an optional per-head sink in the denominator, values that
+    may be the leading ``value_dims`` entries of the cached keys
+    (``v_cache`` None) and an optional sigmoid gate per (row, head) on the
+    result. ``tiles`` as for ranged_paged_attention."""
+    if q.is_cuda:
+        T, H, _ = q.shape
+        V = v_cache.shape[3] if v_cache is not None else int(value_dims)
+        out = torch.empty((T, H, V), dtype=q.dtype, device=q.device)
+        tile_seq = tile_row0 = None
+        tile_rows = 0
+        if tiles is not None and seq_cu is not None and tiles[2] > 0:
+            tile_seq, tile_row0, tile_rows = tiles
+        rest = T - tile_rows
+        part_ml = part_o = None
+        if rest > 0:
+            bs = k_cache.shape[2]
+            ns = _native().sink_attention_splits(seq_bt.shape[1] * bs)
+            part_ml = torch.empty((rest, H, ns, 2), dtype=torch.float32,
+                                  device=q.device)
+            part_o = torch.empty((rest, H, ns, V), dtype=torch.float32,
+                                 device=q.device)
+        _native().sink_paged_attention(out, q, k_cache, v_cache, seq_bt,
+                                       row_seq, positions, float(scale),
+                                       sink, V, out_gate, seq_cu, tile_seq,
+                                       tile_row0, int(tile_rows), part_ml,
+                                       part_o)
+        return out
+    return ref.sink_paged_attention(q, k_cache, v_cache, seq_bt, row_seq,
+                                    positions, scale, sink, value_dims,
+                                    out_gate)
+
+
+def causal_conv_state(x, conv_w, conv_b, conv_state, seq_cu, row_seq,
+                      seq_slots, positions):
+    """fp32 [T, C] causal convolution of x (a column slice is fine) with
+    the per-sequence tail kept in conv_state."""
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+        _native().causal_conv_state(out, x, conv_w, conv_b, conv_state,
+                                    seq_cu, row_seq, seq_slots, positions)
+        return out
+    return ref.causal_conv_state(x, conv_w, conv_b, conv_state, seq_cu,
+                                 seq_slots, positions)
+
+
+def rglru_scan(u, gate_lin, gate_bias, lam, y_lin, state, seq_cu, seq_slots,
+               positions, decay_scale: float, out_dtype, max_rows: int = 0):
+    """Gated linear recurrence over the rows of every group; returns
+    S_t * gelu_tanh(y_lin_t) in out_dtype. ``max_rows``: longest group of
+    the step (0: unknown)."""
+    if u.is_cuda:
+        out = torch.empty(u.shape, dtype=out_dtype, device=u.device)
+        _native().rglru_scan(out, u, gate_lin, gate_bias, lam, y_lin, state,
+                             seq_cu, seq_slots, positions,
+                             float(decay_scale), int(max_rows))
+        return out
+    return ref.rglru_scan(u, gate_lin, gate_bias, lam,
+                          ref.gelu_tanh(y_lin.float()), state, seq_cu,
+                          seq_slots, positions, decay_scale, out_dtype)
+
+
+def relu_squared(x):
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _native().relu_squared(out, x)
+        return out
+    return ref.relu_squared(x)

@@ -412,3 +412,206 @@ def gated_delta_rule(x, conv_w, alin, blin, a_log, dt_bias, conv_state,
         if slot >= 0:
             state[slot] = S
     return o.reshape(T, heads * vdim)
+
+
+# ------------------------------------------------------------------------
+# parallel-residual stream, weighted head norms with a query temperature,
+# latent (low-rank) keys/values with a shared rotated part and a softmax
+# sink, gated linear recurrence behind a short convolution, squared relu.
+
+def scaled_residual_layer_norm_(resid, ys, scales, w_next, eps: float,
+                                out_dtype):
+    """resid += sum_i scales[i] * ys[i] in fp32, in place; optionally
+    returns layer_norm(resid) * w_next."""
+    acc = None
+    for y, s in zip(ys, scales):
+        term = y.float() * s
+        acc = term if acc is None else acc + term
+    resid.add_(acc)
+    if w_next is None:
+        return None
+    return layer_norm(resid, w_next, eps, out_dtype)
+
+
+def query_temperature(positions, coef: float, every: int):
+    """1 + coef * ln(floor((p + 1) / every) + 1) per row, fp32 (1 when
+    every <= 0)."""
+    if every <= 0 or coef == 0.0:
+        return torch.ones(positions.shape[0], dtype=torch.float32)
+    blk = torch.div(positions.long() + 1, every, rounding_mode="floor")
+    return 1.0 + coef * torch.log((blk + 1).float())
+
+
+def headnorm_qtemp_cache_(q, k, v, positions, q_w, k_w, eps: float,
+                          temp_coef: float, temp_every: int, k_cache,
+                          v_cache, slot_mapping, num_heads: int,
+                          num_kv_heads: int, dim: int, vdim: int):
+    """Every query and key head is divided by its root mean square and
+    multiplied by a weight vector shared by all heads (q_w / k_w, [dim]);
+    queries are then multiplied by the position's temperature. Normed keys
+    and the unchanged values go to the paged caches; returns the
+    processed queries [T, H, dim]."""
+    T = q.shape[0]
+    qf = _rms(q.float().reshape(T, num_heads, dim), eps) * q_w.float()
+    kf = _rms(k.float().reshape(T, num_kv_heads, dim), eps) * k_w.float()
+    qf = qf * query_temperature(positions, temp_coef,
+                                temp_every).reshape(T, 1, 1)
+    paged_cache_write_(kf.reshape(T, -1).to(q.dtype), v, k_cache, v_cache,
+                       slot_mapping)
+    return qf.to(q.dtype)
+
+
+def _rotate_interleaved(x, ang):
+    """Pairs (2i, 2i+1) of the last dim of x turned by ang[..., i]."""
+    cs, sn = torch.cos(ang), torch.sin(ang)
+    u, w = x[..., 0::2], x[..., 1::2]
+    out = torch.empty_like(x)
+    out[..., 0::2] = u * cs - w * sn
+    out[..., 1::2] = w * cs + u * sn
+    return out
+
+
+def latent_rope_cache_(q, ckr, positions, inv_freq, norm_w, eps: float,
+                       kv_cache, slot_mapping, num_heads: int, dim: int,
+                       rot_dim: int, rank: int, q_out):
+    """q [T, H*(dim+rot_dim)]: the trailing rot_dim entries of every head
+    are rotated (interleaved pairs, fp32 angle = position * inv_freq) and
+    written to q_out[:, :, rank:]. ckr [T, rank+rot_dim]: the leading rank
+    entries are RMS-normed with norm_w, the trailing rot_dim rotated; the
+    row goes to kv_cache [B, 1, bs, rank+rot_dim] at slot_mapping."""
+    T = q.shape[0]
+    ang = positions.float()[:, None] * inv_freq.float()[None, :]
+    qr = q.float().reshape(T, num_heads, dim + rot_dim)[:, :, dim:]
+    q_out[:, :, rank:] = _rotate_interleaved(qr, ang[:, None, :]).to(
+        q_out.dtype)
+    cf = ckr.float()
+    row = torch.cat([_rms(cf[:, :rank], eps) * norm_w.float(),
+                     _rotate_interleaved(cf[:, rank:], ang)], dim=-1)
+    bs = kv_cache.shape[2]
+    slots = slot_mapping.long()
+    ok = slots >= 0
+    kv_cache[slots[ok] // bs, 0, slots[ok] % bs, :] = row[ok].to(
+        kv_cache.dtype)
+
+
+def sink_paged_attention(q, k_cache, v_cache, seq_bt, row_seq, positions,
+                         scale: float, sink=None, value_dims: int = 0,
+                         out_gate=None):
+    """Causal softmax attention of every row over the paged keys 0..p of
+    its own sequence. ``sink`` [H] fp32: exp(sink_h) joins the softmax
+    denominator (no key, no value). ``v_cache`` None: the values are the
+    leading ``value_dims`` entries of the cached keys. ``out_gate`` [T, H]:
+    head results are multiplied by sigmoid(out_gate). q [T, H, Dk];
+    returns [T, H, Dv]."""
+    T, H, D = q.shape
+    G, bs = k_cache.shape[1], k_cache.shape[2]
+    rep = H // G
+    V = v_cache.shape[3] if v_cache is not None else int(value_dims)
+    out = torch.zeros(T, H, V, dtype=torch.float32)
+    pos = positions.tolist()
+    rs = row_seq.tolist()
+    qf = q.float()
+    t = 0
+    while t < T:
+        s = rs[t]
+        e = t
+        while e + 1 < T and rs[e + 1] == s:
+            e += 1
+        idx = torch.arange(0, pos[e] + 1)
+        blocks = seq_bt[s].long()[idx // bs]
+        kk = k_cache[blocks, :, idx % bs, :].float()   # [L, G, D]
+        vv = (v_cache[blocks, :, idx % bs, :].float() if v_cache is not None
+              else kk[:, :, :V])
+        kk = kk.repeat_interleave(rep, dim=1)
+        vv = vv.repeat_interleave(rep, dim=1)
+        pr = torch.tensor(pos[t:e + 1])
+        sc = torch.einsum("ihd,jhd->hij", qf[t:e + 1], kk) * scale
+        vis = idx[None, :] <= pr[:, None]
+        sc = sc.masked_fill(~vis[None], float("-inf"))
+        m = sc.max(dim=-1, keepdim=True).values
+        if sink is not None:
+            m = torch.maximum(m, sink.float().reshape(H, 1, 1))
+        ex = torch.exp(sc - m)
+        den = ex.sum(dim=-1, keepdim=True)
+        if sink is not None:
+            den = den + torch.exp(sink.float().reshape(H, 1, 1) - m)
+        out[t:e + 1] = torch.einsum("hij,jhd->ihd", ex / den, vv)
+        t = e + 1
+    if out_gate is not None:
+        out = out * torch.sigmoid(out_gate.float()).reshape(T, H, 1)
+    return out.to(q.dtype)
+
+
+def causal_conv_state(x, conv_w, conv_b, conv_state, seq_cu, seq_slots,
+                      positions):
+    """Causal convolution over time per channel with a bias: conv_w
+    [C, taps] (last column = current token), zeros before the sequence
+    start. ``conv_state`` [slots, max(taps-1, 1), C] fp32 keeps each
+    sequence's last taps-1 inputs between steps. Returns fp32 [T, C]."""
+    T, C = x.shape
+    taps = conv_w.shape[1]
+    xf = x.float()
+    wf = conv_w.float()
+    y = torch.empty(T, C, dtype=torch.float32)
+    cu, slots, pos = seq_cu.tolist(), seq_slots.tolist(), positions.tolist()
+    for s in range(len(slots)):
+        a, b = cu[s], cu[s + 1]
+        if b <= a:
+            continue
+        slot, p0 = slots[s], pos[a]
+        hist = torch.zeros(taps - 1, C, dtype=torch.float32)
+        if slot >= 0 and p0 > 0 and taps > 1:
+            hist = conv_state[slot, : taps - 1].clone()
+        ext = torch.cat([hist, xf[a:b]], dim=0)
+        acc = conv_b.float().expand(b - a, C).clone()
+        for j in range(taps):
+            acc += wf[:, j] * ext[j: j + (b - a)]
+        y[a:b] = acc
+        if slot >= 0 and taps > 1:
+            conv_state[slot, : taps - 1] = ext[-(taps - 1):]
+    return y
+
+
+def rglru_scan(u, gate_lin, gate_bias, lam, y, state, seq_cu, seq_slots,
+               positions, decay_scale: float, out_dtype):
+    """Real-gated linear recurrence per channel. u [T, W] fp32; gate_lin
+    [B, T, 2*bw] fp32 (recurrence gate first, input gate second, W = B*bw)
+    plus gate_bias [B, 2*bw]; with r = sigmoid(.), i = sigmoid(.),
+    log a = -decay_scale * r * softplus(lam):
+
+        S_t = a_t S_(t-1) + sqrt(1 - a_t^2) i_t u_t,   out_t = S_t * y_t.
+
+    ``state`` [slots, W] fp32 carries S (zero at position 0)."""
+    T, W = u.shape
+    B = gate_lin.shape[0]
+    bw = W // B
+    g = gate_lin.float() + gate_bias.float()[:, None, :]
+    r = torch.sigmoid(g[:, :, :bw]).permute(1, 0, 2).reshape(T, W)
+    i = torch.sigmoid(g[:, :, bw:]).permute(1, 0, 2).reshape(T, W)
+    log_a = -decay_scale * r * torch.nn.functional.softplus(lam.float())
+    a = torch.exp(log_a)
+    b_in = torch.sqrt(-torch.expm1(2.0 * log_a)) * i * u.float()
+    out = torch.empty(T, W, dtype=torch.float32)
+    cu, slots, pos = seq_cu.tolist(), seq_slots.tolist(), positions.tolist()
+    for s in range(len(slots)):
+        t0, t1 = cu[s], cu[s + 1]
+        if t1 <= t0:
+            continue
+        S = _group_state(state, slots[s], pos[t0], (W,))
+        for t in range(t0, t1):
+            S = a[t] * S + b_in[t]
+            out[t] = S
+        if slots[s] >= 0:
+            state[slots[s]] = S
+    return (out * y.float()).to(out_dtype)
+
+
+def gelu_tanh(x):
+    xf = x.float()
+    return (0.5 * xf * (1.0 + torch.tanh(
+        math.sqrt(2.0 / math.pi) * (xf + 0.044715 * xf.pow(3))))).to(x.dtype)
+
+
+def relu_squared(x):
+    xf = torch.relu(x.float())
+    return (xf * xf).to(x.dtype)
