@@ -49,6 +49,8 @@ SEQMIX_SOURCES = [
     "seqmix_stream.hip",
     "seqmix_linear.hip",
     "seqmix_window.hip",
+    "seqmix_parallel.hip",
+    "seqmix_sink.hip",
 ]
 
 EXTENSIONS = {

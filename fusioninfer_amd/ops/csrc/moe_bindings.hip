@@ -13,7 +13,7 @@
 namespace fi {
 
 void launch_moe_gemm(u16*, const u16*, const u16*, const int*, const int*,
-                     const int*, int, int, int, int, bool, hipStream_t);
+                     const int*, int, int, int, int, int, hipStream_t);
 void launch_moe_gemm_fp8(u16*, const unsigned char*, const float*,
                          const unsigned char*, const float*, const int*,
                          const int*, const int*, int, int, int, int, bool,
@@ -29,7 +29,7 @@ void launch_moe_combine(A*, const A*, const int*, const float*, int, int,
                         int, hipStream_t);
 template <typename A>
 void launch_moe_gemm_plain(A*, const A*, const A*, const int*, const int*,
-                           const int*, int, int, int, int, bool, hipStream_t);
+                           const int*, int, int, int, int, int, hipStream_t);
 
 }  // namespace fi
 
@@ -52,7 +52,11 @@ hipStream_t current_stream() {
 
 void moe_gemm(at::Tensor out, at::Tensor a, at::Tensor b_packed,
               at::Tensor sorted_ids, at::Tensor expert_ids,
-              at::Tensor n_valid, int64_t block_m, bool gate_up) {
+              at::Tensor n_valid, int64_t block_m, int64_t mode) {
+  // mode 0: plain; 1: gathered rows, silu(gate) * up; 2: gathered rows,
+  // relu(up)^2
+  TORCH_CHECK(mode >= 0 && mode <= 2, "unknown grouped GEMM mode");
+  const bool gate_up = mode == 1;
   CHECK_BF16_CUDA(out);
   CHECK_BF16_CUDA(a);
   CHECK_BF16_CUDA(b_packed);
@@ -68,7 +72,7 @@ void moe_gemm(at::Tensor out, at::Tensor a, at::Tensor b_packed,
   TORCH_CHECK(PM % block_m == 0, "padded rows must be block_m-aligned");
   TORCH_CHECK(K % 32 == 0, "K must be a multiple of 32");
   TORCH_CHECK(
-      N % (block_m == 16 ? 64 : (gate_up ? 64 : 128)) == 0,
+      N % (block_m == 16 ? 64 : (mode != 0 ? 64 : 128)) == 0,
       "N tile misalignment");
   // packed B: [E, K/32, NB/16, 64, 8]
   TORCH_CHECK(b_packed.dim() == 5 && b_packed.size(1) == K / 32 &&
@@ -76,11 +80,13 @@ void moe_gemm(at::Tensor out, at::Tensor a, at::Tensor b_packed,
               b_packed.size(3) == 64 && b_packed.size(4) == 8,
               "b_packed layout mismatch");
   TORCH_CHECK(expert_ids.size(0) >= PM / block_m);
-  if (gate_up) TORCH_CHECK(sorted_ids.size(0) >= PM);
+  if (mode != 0) TORCH_CHECK(sorted_ids.size(0) >= PM);
+  if (mode == 0) TORCH_CHECK(a.size(0) >= PM);
   fi::launch_moe_gemm(bf16_ptr(out), bf16_cptr(a),
                       bf16_cptr(b_packed), sorted_ids.data_ptr<int>(),
                       expert_ids.data_ptr<int>(), n_valid.data_ptr<int>(),
-                      PM / block_m, K, N, static_cast<int>(block_m), gate_up,
+                      PM / block_m, K, N, static_cast<int>(block_m),
+                      static_cast<int>(mode),
                       current_stream());
 }
 
@@ -145,7 +151,9 @@ void moe_combine(at::Tensor out, at::Tensor y, at::Tensor pos, at::Tensor w) {
 
 void moe_gemm_plain(at::Tensor out, at::Tensor a, at::Tensor w,
                     at::Tensor sorted_ids, at::Tensor expert_ids,
-                    at::Tensor n_valid, int64_t block_m, bool gate_up) {
+                    at::Tensor n_valid, int64_t block_m, int64_t mode) {
+  TORCH_CHECK(mode >= 0 && mode <= 2, "unknown grouped GEMM mode");
+  const bool gate_up = mode == 1;
   TORCH_CHECK(out.is_cuda() && a.is_cuda() && w.is_cuda());
   TORCH_CHECK(out.scalar_type() == a.scalar_type() &&
               out.scalar_type() == w.scalar_type() &&
@@ -163,19 +171,19 @@ void moe_gemm_plain(at::Tensor out, at::Tensor a, at::Tensor w,
               w.size(1) == (gate_up ? 2 * N : N), "expert weight shape");
   TORCH_CHECK(expert_ids.size(0) >= PM / block_m);
   TORCH_CHECK(sorted_ids.size(0) >= PM);
-  if (!gate_up) TORCH_CHECK(a.size(0) == PM);
+  if (mode == 0) TORCH_CHECK(a.size(0) == PM);
   if (PM == 0) return;
   if (out.scalar_type() == at::kBFloat16)
     fi::launch_moe_gemm_plain<u16>(
         bf16_ptr(out), bf16_cptr(a), bf16_cptr(w), sorted_ids.data_ptr<int>(),
         expert_ids.data_ptr<int>(), n_valid.data_ptr<int>(), PM, K, N,
-        static_cast<int>(block_m), gate_up, current_stream());
+        static_cast<int>(block_m), static_cast<int>(mode), current_stream());
   else
     fi::launch_moe_gemm_plain<float>(
         out.data_ptr<float>(), a.data_ptr<float>(), w.data_ptr<float>(),
         sorted_ids.data_ptr<int>(), expert_ids.data_ptr<int>(),
-        n_valid.data_ptr<int>(), PM, K, N, static_cast<int>(block_m), gate_up,
-        current_stream());
+        n_valid.data_ptr<int>(), PM, K, N, static_cast<int>(block_m),
+        static_cast<int>(mode), current_stream());
 }
 
 void moe_route(at::Tensor logits, at::Tensor topv, at::Tensor topi, int64_t k,

@@ -58,7 +58,7 @@ FI_DEV short8 load_b16x8(const u16* p) {
 // per K-step — the guide's 2-phase grouped-GEMM shape), so the four
 // waves share one gather of the 128x32 panel instead of issuing
 // per-wave fragment loads against L2/L3.
-template <int WM, int WN, int MITER, int NITER, bool GATE_UP,
+template <int WM, int WN, int MITER, int NITER, int MODE,
           bool STAGE_A = false>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(
     u16* __restrict__ out,              // [PM, N] bf16
@@ -68,6 +68,10 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
     const int* __restrict__ expert_ids, // [PM/BM] local expert per m-tile
     const int* __restrict__ n_valid,    // device scalar: real m-tile count
     const int K, const int N) {
+  // MODE 0: plain GEMM over act rows; 1: gathered x rows, gate|up
+  // columns, silu(gate) * up; 2: gathered x rows, up alone, relu(up)^2
+  constexpr bool GATE_UP = MODE == 1;
+  constexpr bool GATHER = MODE != 0;
   constexpr int BM = 16 * WM * MITER;
   static_assert(!STAGE_A || BM == 128, "STAGE_A is tuned for BM=128");
   const int mtile = blockIdx.x;
@@ -103,7 +107,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
 #pragma unroll
   for (int mi = 0; mi < MITER; ++mi) {
     const int slot = row0 + mi * 16 + (lane & 15);
-    const int row = GATE_UP ? sorted_ids[slot] : slot;
+    const int row = GATHER ? sorted_ids[slot] : slot;
     a_p[mi] = a + static_cast<int64_t>(row) * K + (lane >> 4) * 8;
   }
 
@@ -124,7 +128,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
       const int X = (i * 256 + tid) * 16;       // linear LDS byte
       const int srow = X / kARowB;
       const int sbyte = (X % kARowB) ^ ((srow & 3) << 4);
-      const int gr = GATE_UP ? sorted_ids[mtile * BM + srow]
+      const int gr = GATHER ? sorted_ids[mtile * BM + srow]
                              : mtile * BM + srow;
       stage_row_off[i] = static_cast<int64_t>(gr) * K;
       stage_src_off[i] = sbyte / 2;
@@ -257,6 +261,10 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
           v = (g / (1.f + __expf(-g))) * u;
         } else {
           v = acc_g[mi][ni][r];
+          if (MODE == 2) {
+            v = fmaxf(v, 0.f);
+            v *= v;
+          }
         }
         out[static_cast<int64_t>(orow) * N + col] = f32_to_bf16(v);
       }
@@ -478,15 +486,19 @@ __global__ __launch_bounds__(256) void moe_gemm_fp8_kernel(
 void launch_moe_gemm(u16* out, const u16* a, const u16* b,
                      const int* sorted_ids, const int* expert_ids,
                      const int* n_valid, int max_mtiles, int K, int N,
-                     int block_m, bool gate_up, hipStream_t stream) {
+                     int block_m, int mode, hipStream_t stream) {
   if (block_m == 16) {
     const dim3 grid(max_mtiles, N / 64);
-    if (gate_up)
-      hipLaunchKernelGGL((moe_gemm_kernel<1, 4, 1, 1, true>), grid, dim3(256),
+    if (mode == 1)
+      hipLaunchKernelGGL((moe_gemm_kernel<1, 4, 1, 1, 1>), grid, dim3(256),
+                         0, stream, out, a, b, sorted_ids, expert_ids,
+                         n_valid, K, N);
+    else if (mode == 2)
+      hipLaunchKernelGGL((moe_gemm_kernel<1, 4, 1, 1, 2>), grid, dim3(256),
                          0, stream, out, a, b, sorted_ids, expert_ids,
                          n_valid, K, N);
     else
-      hipLaunchKernelGGL((moe_gemm_kernel<1, 4, 1, 1, false>), grid,
+      hipLaunchKernelGGL((moe_gemm_kernel<1, 4, 1, 1, 0>), grid,
                          dim3(256), 0, stream, out, a, b, sorted_ids,
                          expert_ids, n_valid, K, N);
   } else {  // block_m == 128
@@ -495,24 +507,34 @@ void launch_moe_gemm(u16* out, const u16* a, const u16* b,
       const char* e = getenv("FI_MOE_STAGE_A");
       return !(e && e[0] == '0');
     }();
-    if (gate_up) {
+    if (mode == 1) {
       const dim3 grid(max_mtiles, N / 64);
       if (stage_a)
-        hipLaunchKernelGGL((moe_gemm_kernel<2, 2, 4, 2, true, true>), grid,
+        hipLaunchKernelGGL((moe_gemm_kernel<2, 2, 4, 2, 1, true>), grid,
                            dim3(256), 0, stream, out, a, b, sorted_ids,
                            expert_ids, n_valid, K, N);
       else
-        hipLaunchKernelGGL((moe_gemm_kernel<2, 2, 4, 2, true, false>), grid,
+        hipLaunchKernelGGL((moe_gemm_kernel<2, 2, 4, 2, 1, false>), grid,
+                           dim3(256), 0, stream, out, a, b, sorted_ids,
+                           expert_ids, n_valid, K, N);
+    } else if (mode == 2) {
+      const dim3 grid(max_mtiles, N / 64);
+      if (stage_a)
+        hipLaunchKernelGGL((moe_gemm_kernel<2, 2, 4, 2, 2, true>), grid,
+                           dim3(256), 0, stream, out, a, b, sorted_ids,
+                           expert_ids, n_valid, K, N);
+      else
+        hipLaunchKernelGGL((moe_gemm_kernel<2, 2, 4, 2, 2, false>), grid,
                            dim3(256), 0, stream, out, a, b, sorted_ids,
                            expert_ids, n_valid, K, N);
     } else {
       const dim3 grid(max_mtiles, N / 128);
       if (stage_a)
-        hipLaunchKernelGGL((moe_gemm_kernel<2, 2, 4, 4, false, true>), grid,
+        hipLaunchKernelGGL((moe_gemm_kernel<2, 2, 4, 4, 0, true>), grid,
                            dim3(256), 0, stream, out, a, b, sorted_ids,
                            expert_ids, n_valid, K, N);
       else
-        hipLaunchKernelGGL((moe_gemm_kernel<2, 2, 4, 4, false, false>), grid,
+        hipLaunchKernelGGL((moe_gemm_kernel<2, 2, 4, 4, 0, false>), grid,
                            dim3(256), 0, stream, out, a, b, sorted_ids,
                            expert_ids, n_valid, K, N);
     }

@@ -10,8 +10,10 @@
 //    (same layout as the MFMA kernel: sorted_ids / expert_ids / n_valid)
 //    on the experts' natural [E, out, in] weights, bf16 or fp32 operands,
 //    fp32 accumulation, any K and N. 16 rows x 64 columns per workgroup,
-//    operands staged through LDS as fp32. gate_up applies
-//    silu(gate) * up on the way out.
+//    operands staged through LDS as fp32. Mode 0: plain GEMM over act
+//    rows; 1: x rows gathered through sorted_ids, gate|up columns,
+//    silu(gate) * up on the way out; 2: gathered x rows, up columns
+//    alone, relu(up)^2 on the way out.
 //  * moe_combine: out[t] = sum_k w[t,k] * y[pos[t,k]], any width, bf16 or
 //    fp32 rows, no atomics.
 
@@ -99,7 +101,7 @@ constexpr int kPlainBM = 16;   // rows per workgroup
 constexpr int kPlainBN = 64;   // columns per workgroup
 constexpr int kPlainKT = 32;   // K step
 
-template <typename A, bool GATE_UP>
+template <typename A, int MODE>
 __global__ __launch_bounds__(256) void moe_gemm_plain_kernel(
     A* __restrict__ out,                // [PM, N]
     const A* __restrict__ a,            // GATE_UP: x [T, K]; else act [PM, K]
@@ -107,6 +109,8 @@ __global__ __launch_bounds__(256) void moe_gemm_plain_kernel(
     const int* __restrict__ sorted_ids, const int* __restrict__ expert_ids,
     const int* __restrict__ n_valid, const int K, const int N,
     const int block_m) {
+  constexpr bool GATE_UP = MODE == 1;
+  constexpr bool GATHER = MODE != 0;
   // m-tiles are block_m rows; this workgroup covers 16 of them
   const int sub = block_m / kPlainBM;
   const int mtile = blockIdx.x / sub;
@@ -122,7 +126,7 @@ __global__ __launch_bounds__(256) void moe_gemm_plain_kernel(
   __shared__ int rows[kPlainBM];
   const int tid = threadIdx.x;
   if (tid < kPlainBM)
-    rows[tid] = GATE_UP ? sorted_ids[row0 + tid] : row0 + tid;
+    rows[tid] = GATHER ? sorted_ids[row0 + tid] : row0 + tid;
   __syncthreads();
 
   const int r = tid / 16;        // output row 0..15
@@ -168,6 +172,9 @@ __global__ __launch_bounds__(256) void moe_gemm_plain_kernel(
     if (GATE_UP) {
       const float g = acc[j];
       v = g / (1.0f + expf(-g)) * acc2[j];
+    } else if (MODE == 2) {
+      v = fmaxf(v, 0.f);
+      v *= v;
     }
     Act<A>::st(out + static_cast<int64_t>(row0 + r) * N + c, v);
   }
@@ -203,14 +210,18 @@ template <typename A>
 void launch_moe_gemm_plain(A* out, const A* a, const A* w,
                            const int* sorted_ids, const int* expert_ids,
                            const int* n_valid, int PM, int K, int N,
-                           int block_m, bool gate_up, hipStream_t stream) {
+                           int block_m, int mode, hipStream_t stream) {
   const dim3 grid(PM / kPlainBM, ceil_div(N, kPlainBN));
-  if (gate_up)
-    hipLaunchKernelGGL((moe_gemm_plain_kernel<A, true>), grid, dim3(256), 0,
+  if (mode == 1)
+    hipLaunchKernelGGL((moe_gemm_plain_kernel<A, 1>), grid, dim3(256), 0,
+                       stream, out, a, w, sorted_ids, expert_ids, n_valid, K,
+                       N, block_m);
+  else if (mode == 2)
+    hipLaunchKernelGGL((moe_gemm_plain_kernel<A, 2>), grid, dim3(256), 0,
                        stream, out, a, w, sorted_ids, expert_ids, n_valid, K,
                        N, block_m);
   else
-    hipLaunchKernelGGL((moe_gemm_plain_kernel<A, false>), grid, dim3(256), 0,
+    hipLaunchKernelGGL((moe_gemm_plain_kernel<A, 0>), grid, dim3(256), 0,
                        stream, out, a, w, sorted_ids, expert_ids, n_valid, K,
                        N, block_m);
 }
@@ -226,7 +237,7 @@ void launch_moe_combine(A* out, const A* y, const int* pos, const float* w,
 #define FI_INST(A)                                                            \
   template void launch_moe_gemm_plain<A>(A*, const A*, const A*, const int*,  \
                                          const int*, const int*, int, int,    \
-                                         int, int, bool, hipStream_t);        \
+                                         int, int, int, hipStream_t);         \
   template void launch_moe_combine<A>(A*, const A*, const int*, const float*, \
                                       int, int, int, hipStream_t);
 FI_INST(float)

@@ -2,6 +2,7 @@
 // Every entry checks operand shapes against what its kernel and grid
 // assume before launching.
 
+#include <algorithm>
 #include <torch/extension.h>
 
 #include <c10/hip/HIPStream.h>
@@ -93,6 +94,48 @@ void launch_talking_window_rows(A*, const A*, int64_t, const A*, const A*,
                                 const float*, const float*, const float*, int,
                                 int, int, int, int, int, int, float, int,
                                 float*, float*, int, hipStream_t);
+template <typename A>
+void launch_scaled_residual_layer_norm(float*, const A*, float, const A*,
+                                       float, const A*, float, const float*,
+                                       A*, float, int, int, hipStream_t);
+template <typename A>
+void launch_headnorm_qtemp_cache(A*, const A*, int64_t, const A*, int64_t,
+                                 const A*, int64_t, const int*, const float*,
+                                 const float*, float, float, int, A*, A*,
+                                 const int*, int, int, int, int, int, int,
+                                 hipStream_t);
+template <typename A>
+void launch_latent_rope_cache(A*, const A*, int64_t, const A*, int64_t,
+                              const int*, const float*, const float*, float,
+                              A*, const int*, int, int, int, int, int, int,
+                              hipStream_t);
+template <typename A>
+void launch_causal_conv_state(float*, const A*, int64_t, const float*,
+                              const float*, float*, const int*, const int*,
+                              const int*, const int*, int, int, int, int, int,
+                              hipStream_t);
+template <typename A>
+void launch_rglru_scan(A*, const float*, const float*, const float*,
+                       const float*, const A*, int64_t, float*, const int*,
+                       const int*, const int*, int, int, int, int, float,
+                       hipStream_t);
+template <typename A>
+void launch_relu_squared(A*, const A*, int64_t, int, int, hipStream_t);
+int sink_attention_splits(int max_keys);
+bool sink_attention_has_tiles(int DK, int DV);
+template <typename A>
+bool launch_sink_attention_tiles(A*, const A*, const A*, const A*, int,
+                                 const int*, int, const int*, const int*,
+                                 const int*, const int*, int, const float*,
+                                 const A*, int64_t, int, int, int, int, int,
+                                 float, hipStream_t);
+template <typename A>
+void launch_sink_attention_rows(A*, float*, float*, const A*, const A*,
+                                const A*, int, const int*, int, const int*,
+                                const int*, const float*, const A*, int64_t,
+                                int, int, int, int, int, int, int, float, int,
+                                hipStream_t);
+
 }  // namespace fi
 
 namespace {
@@ -725,7 +768,337 @@ void talking_window_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
 
 }  // namespace
 
+// ------------------------------------------------------------------------
+// parallel-residual stream, weighted head norms with a query temperature,
+// latent keys/values with a softmax sink, gated linear recurrence
+
+void scaled_residual_layer_norm(at::Tensor resid, at::Tensor y1, double s1,
+                                c10::optional<at::Tensor> y2, double s2,
+                                c10::optional<at::Tensor> y3, double s3,
+                                c10::optional<at::Tensor> w_next,
+                                c10::optional<at::Tensor> out, double eps) {
+  CHECK_F32(resid);
+  CHECK_ACT(y1);
+  TORCH_CHECK(resid.dim() == 2);
+  const int64_t T = resid.size(0), W = resid.size(1);
+  TORCH_CHECK(y1.sizes() == resid.sizes() && y1.is_contiguous());
+  auto opt = [&](const c10::optional<at::Tensor>& y) -> void* {
+    if (!y.has_value()) return nullptr;
+    TORCH_CHECK(y->is_cuda() && y->scalar_type() == y1.scalar_type() &&
+                y->sizes() == resid.sizes() && y->is_contiguous());
+    return y->data_ptr();
+  };
+  void* y2p = opt(y2);
+  void* y3p = opt(y3);
+  TORCH_CHECK(w_next.has_value() == out.has_value());
+  const float* wn = nullptr;
+  void* op = nullptr;
+  if (w_next.has_value()) {
+    CHECK_F32(*w_next);
+    TORCH_CHECK(w_next->numel() == W);
+    TORCH_CHECK(out->is_cuda() && out->scalar_type() == y1.scalar_type() &&
+                out->sizes() == resid.sizes() && out->is_contiguous());
+    wn = w_next->data_ptr<float>();
+    op = out->data_ptr();
+  }
+  DISPATCH_ACT(y1, fi::launch_scaled_residual_layer_norm<A>(
+                       resid.data_ptr<float>(), ptr<A>(y1), (float)s1,
+                       reinterpret_cast<const A*>(y2p), (float)s2,
+                       reinterpret_cast<const A*>(y3p), (float)s3, wn,
+                       reinterpret_cast<A*>(op), (float)eps, (int)T, (int)W,
+                       stream()));
+}
+
+void headnorm_qtemp_cache(at::Tensor q_out, at::Tensor q, at::Tensor k,
+                          at::Tensor v, at::Tensor positions, at::Tensor q_w,
+                          at::Tensor k_w, double eps, double coef,
+                          int64_t every, at::Tensor k_cache,
+                          at::Tensor v_cache, at::Tensor slot_mapping,
+                          int64_t H, int64_t G, int64_t D, int64_t V) {
+  CHECK_ACT(q);
+  CHECK_ACT(k);
+  CHECK_ACT(v);
+  CHECK_ACT(q_out);
+  CHECK_I32(positions);
+  CHECK_I32(slot_mapping);
+  CHECK_F32(q_w);
+  CHECK_F32(k_w);
+  const int64_t T = q.size(0);
+  check_rows(q, T, H * D, "q");
+  check_rows(k, T, G * D, "k");
+  check_rows(v, T, G * V, "v");
+  const auto dt = q.scalar_type();
+  TORCH_CHECK(k.scalar_type() == dt && v.scalar_type() == dt &&
+              q_out.scalar_type() == dt);
+  TORCH_CHECK(q_out.is_contiguous() && q_out.numel() == T * H * D);
+  TORCH_CHECK(positions.numel() == T && slot_mapping.numel() == T);
+  TORCH_CHECK(q_w.numel() == D && k_w.numel() == D);
+  TORCH_CHECK(k_cache.is_cuda() && v_cache.is_cuda() &&
+              k_cache.is_contiguous() && v_cache.is_contiguous() &&
+              k_cache.scalar_type() == dt && v_cache.scalar_type() == dt);
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 &&
+              k_cache.size(0) == v_cache.size(0) && k_cache.size(1) == G &&
+              v_cache.size(1) == G && k_cache.size(2) == v_cache.size(2) &&
+              k_cache.size(3) == D && v_cache.size(3) == V);
+  TORCH_CHECK(D >= 1 && D <= 512 && V >= 1, "head size out of range");
+  DISPATCH_ACT(q, fi::launch_headnorm_qtemp_cache<A>(
+                      ptr<A>(q_out), ptr<A>(q), q.stride(0), ptr<A>(k),
+                      k.stride(0), ptr<A>(v), v.stride(0),
+                      positions.data_ptr<int>(), q_w.data_ptr<float>(),
+                      k_w.data_ptr<float>(), (float)eps, (float)coef,
+                      (int)every, ptr<A>(k_cache), ptr<A>(v_cache),
+                      slot_mapping.data_ptr<int>(), (int)T, (int)H, (int)G,
+                      (int)D, (int)V, (int)k_cache.size(2), stream()));
+}
+
+void latent_rope_cache(at::Tensor q_out, at::Tensor q, at::Tensor ckr,
+                       at::Tensor positions, at::Tensor inv_freq,
+                       at::Tensor norm_w, double eps, at::Tensor kv_cache,
+                       at::Tensor slot_mapping, int64_t H, int64_t D,
+                       int64_t R, int64_t C) {
+  CHECK_ACT(q);
+  CHECK_ACT(ckr);
+  CHECK_ACT(q_out);
+  CHECK_I32(positions);
+  CHECK_I32(slot_mapping);
+  CHECK_F32(inv_freq);
+  CHECK_F32(norm_w);
+  const int64_t T = q.size(0);
+  check_rows(q, T, H * (D + R), "q");
+  check_rows(ckr, T, C + R, "latent projection");
+  const auto dt = q.scalar_type();
+  TORCH_CHECK(ckr.scalar_type() == dt && q_out.scalar_type() == dt);
+  TORCH_CHECK(q_out.is_contiguous() && q_out.dim() == 3 &&
+              q_out.size(0) == T && q_out.size(1) == H &&
+              q_out.size(2) == C + R);
+  TORCH_CHECK(positions.numel() == T && slot_mapping.numel() == T);
+  TORCH_CHECK(R % 2 == 0 && inv_freq.numel() == R / 2 && norm_w.numel() == C);
+  TORCH_CHECK(kv_cache.is_cuda() && kv_cache.is_contiguous() &&
+              kv_cache.scalar_type() == dt && kv_cache.dim() == 4 &&
+              kv_cache.size(1) == 1 && kv_cache.size(3) == C + R);
+  DISPATCH_ACT(q, fi::launch_latent_rope_cache<A>(
+                      ptr<A>(q_out), ptr<A>(q), q.stride(0), ptr<A>(ckr),
+                      ckr.stride(0), positions.data_ptr<int>(),
+                      inv_freq.data_ptr<float>(), norm_w.data_ptr<float>(),
+                      (float)eps, ptr<A>(kv_cache),
+                      slot_mapping.data_ptr<int>(), (int)T, (int)H, (int)D,
+                      (int)R, (int)C, (int)kv_cache.size(2), stream()));
+}
+
+int64_t sink_attention_splits(int64_t max_keys) {
+  return fi::sink_attention_splits((int)max_keys);
+}
+
+bool sink_attention_has_tiles(int64_t DK, int64_t DV) {
+  return fi::sink_attention_has_tiles((int)DK, (int)DV);
+}
+
+// Rows [0, tile_rows) belong to the row groups that the tile tables cover
+// and run the MFMA kernel when the sizes have one; all other rows run the
+// split form, part_ml.size(0) rows per launch.
+void sink_paged_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
+                          c10::optional<at::Tensor> v_cache,
+                          at::Tensor seq_bt, at::Tensor row_seq,
+                          at::Tensor positions, double scale,
+                          c10::optional<at::Tensor> sink, int64_t DV,
+                          c10::optional<at::Tensor> gate,
+                          c10::optional<at::Tensor> seq_cu,
+                          c10::optional<at::Tensor> tile_seq,
+                          c10::optional<at::Tensor> tile_row0,
+                          int64_t tile_rows,
+                          c10::optional<at::Tensor> part_ml,
+                          c10::optional<at::Tensor> part_o) {
+  CHECK_ACT(q);
+  CHECK_ACT(out);
+  CHECK_I32(row_seq);
+  CHECK_I32(positions);
+  TORCH_CHECK(seq_bt.is_cuda() && seq_bt.scalar_type() == at::kInt &&
+              seq_bt.dim() == 2 && seq_bt.stride(1) == 1);
+  TORCH_CHECK(q.dim() == 3 && q.is_contiguous() && out.is_contiguous() &&
+              out.scalar_type() == q.scalar_type());
+  const int T = q.size(0), H = q.size(1), DK = q.size(2);
+  const auto dt = q.scalar_type();
+  TORCH_CHECK(k_cache.is_cuda() && k_cache.is_contiguous() &&
+              k_cache.scalar_type() == dt && k_cache.dim() == 4 &&
+              k_cache.size(3) == DK);
+  const int G = k_cache.size(1), bs = k_cache.size(2);
+  const void* vp = k_cache.data_ptr();
+  int v_row = DK;
+  if (v_cache.has_value()) {
+    TORCH_CHECK(v_cache->is_cuda() && v_cache->is_contiguous() &&
+                v_cache->scalar_type() == dt && v_cache->dim() == 4 &&
+                v_cache->size(0) == k_cache.size(0) &&
+                v_cache->size(1) == G && v_cache->size(2) == bs &&
+                v_cache->size(3) == DV);
+    vp = v_cache->data_ptr();
+    v_row = DV;
+  } else {
+    TORCH_CHECK(DV >= 1 && DV <= DK, "value slice exceeds the key row");
+  }
+  TORCH_CHECK(out.dim() == 3 && out.size(0) == T && out.size(1) == H &&
+              out.size(2) == DV);
+  TORCH_CHECK(G >= 1 && H % G == 0 && DK >= 1 && DK <= 1024 && DV >= 1);
+  TORCH_CHECK(row_seq.numel() == T && positions.numel() == T);
+  const float* sp = nullptr;
+  if (sink.has_value()) {
+    CHECK_F32(*sink);
+    TORCH_CHECK(sink->numel() == H);
+    sp = sink->data_ptr<float>();
+  }
+  const void* gp = nullptr;
+  int64_t g_stride = 0;
+  if (gate.has_value()) {
+    TORCH_CHECK(gate->is_cuda() && gate->scalar_type() == dt);
+    check_rows(*gate, T, H, "output gate");
+    gp = gate->data_ptr();
+    g_stride = gate->stride(0);
+  }
+  TORCH_CHECK(tile_rows >= 0 && tile_rows <= T);
+  int64_t done = 0;
+  if (tile_rows > 0) {
+    TORCH_CHECK(seq_cu.has_value() && tile_seq.has_value() &&
+                tile_row0.has_value());
+    CHECK_I32(*seq_cu);
+    CHECK_I32(*tile_seq);
+    CHECK_I32(*tile_row0);
+    TORCH_CHECK(tile_seq->numel() == tile_row0->numel());
+    TORCH_CHECK(seq_cu->numel() <= seq_bt.size(0) + 1);
+    bool ok = false;
+    DISPATCH_ACT(q, ok = fi::launch_sink_attention_tiles<A>(
+                      ptr<A>(out), ptr<A>(q), ptr<A>(k_cache),
+                      reinterpret_cast<const A*>(vp), v_row,
+                      seq_bt.data_ptr<int>(), (int)seq_bt.stride(0),
+                      seq_cu->data_ptr<int>(), positions.data_ptr<int>(),
+                      tile_seq->data_ptr<int>(), tile_row0->data_ptr<int>(),
+                      (int)tile_seq->numel(), sp,
+                      reinterpret_cast<const A*>(gp), g_stride, H, G, DK,
+                      (int)DV, bs, (float)scale, stream()));
+    if (ok) done = tile_rows;
+  }
+  if (done == T) return;
+  TORCH_CHECK(part_ml.has_value() && part_o.has_value(),
+              "rows outside the tiled form need the span buffers");
+  CHECK_F32(*part_ml);
+  CHECK_F32(*part_o);
+  const int ns = fi::sink_attention_splits((int)seq_bt.size(1) * bs);
+  TORCH_CHECK(part_ml->dim() == 4 && part_o->dim() == 4 &&
+              part_ml->size(0) >= 1 && part_o->size(0) == part_ml->size(0) &&
+              part_ml->size(1) == H && part_ml->size(2) == ns &&
+              part_ml->size(3) == 2 && part_o->size(1) == H &&
+              part_o->size(2) == ns && part_o->size(3) == DV);
+  const int cap = part_ml->size(0);
+  for (int row0 = (int)done; row0 < T; row0 += cap) {
+    const int rows = std::min(cap, T - row0);
+    DISPATCH_ACT(q, fi::launch_sink_attention_rows<A>(
+                        ptr<A>(out), part_ml->data_ptr<float>(),
+                        part_o->data_ptr<float>(), ptr<A>(q), ptr<A>(k_cache),
+                        reinterpret_cast<const A*>(vp), v_row,
+                        seq_bt.data_ptr<int>(), (int)seq_bt.stride(0),
+                        row_seq.data_ptr<int>(), positions.data_ptr<int>(),
+                        sp, reinterpret_cast<const A*>(gp), g_stride, row0,
+                        rows, H, G, DK, (int)DV, bs, (float)scale, ns,
+                        stream()));
+  }
+}
+
+void causal_conv_state(at::Tensor out, at::Tensor x, at::Tensor conv_w,
+                       at::Tensor conv_b, at::Tensor conv_state,
+                       at::Tensor seq_cu, at::Tensor row_seq,
+                       at::Tensor seq_slots, at::Tensor positions) {
+  CHECK_F32(out);
+  CHECK_ACT(x);
+  CHECK_F32(conv_w);
+  CHECK_F32(conv_b);
+  CHECK_F32(conv_state);
+  CHECK_I32(seq_cu);
+  CHECK_I32(row_seq);
+  CHECK_I32(positions);
+  const int64_t T = x.size(0), C = x.size(1);
+  check_rows(x, T, C, "convolution input");
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == C);
+  TORCH_CHECK(conv_w.dim() == 2 && conv_w.size(0) == C && conv_b.numel() == C);
+  const int taps = conv_w.size(1);
+  TORCH_CHECK(taps >= 1 && taps <= 64);
+  TORCH_CHECK(conv_state.dim() == 3 && conv_state.size(2) == C &&
+              conv_state.size(1) >= std::max(taps - 1, 1));
+  check_groups(seq_cu, seq_slots, positions, T);
+  TORCH_CHECK(row_seq.numel() == T && positions.numel() == T);
+  const int S = seq_slots.numel();
+  DISPATCH_ACT(x, fi::launch_causal_conv_state<A>(
+                      out.data_ptr<float>(), ptr<A>(x), x.stride(0),
+                      conv_w.data_ptr<float>(), conv_b.data_ptr<float>(),
+                      conv_state.data_ptr<float>(), seq_cu.data_ptr<int>(),
+                      row_seq.data_ptr<int>(), seq_slots.data_ptr<int>(),
+                      positions.data_ptr<int>(), (int)T, S, (int)C, taps,
+                      (int)conv_state.size(1), stream()));
+}
+
+void rglru_scan(at::Tensor out, at::Tensor u, at::Tensor gate_lin,
+                at::Tensor gate_bias, at::Tensor lam, at::Tensor y_lin,
+                at::Tensor state, at::Tensor seq_cu, at::Tensor seq_slots,
+                at::Tensor positions, double decay_scale, int64_t max_rows) {
+  CHECK_ACT(out);
+  CHECK_F32(u);
+  CHECK_F32(gate_lin);
+  CHECK_F32(gate_bias);
+  CHECK_F32(lam);
+  CHECK_ACT(y_lin);
+  CHECK_F32(state);
+  CHECK_I32(positions);
+  const int64_t T = u.size(0), W = u.size(1);
+  TORCH_CHECK(u.dim() == 2 && out.is_contiguous() && out.dim() == 2 &&
+              out.size(0) == T && out.size(1) == W &&
+              out.scalar_type() == y_lin.scalar_type());
+  check_rows(y_lin, T, W, "gelu branch");
+  TORCH_CHECK(gate_lin.dim() == 3 && gate_lin.size(1) == T);
+  const int64_t B = gate_lin.size(0);
+  TORCH_CHECK(B >= 1 && W % B == 0 && gate_lin.size(2) == 2 * (W / B));
+  TORCH_CHECK(gate_bias.numel() == 2 * W && lam.numel() == W);
+  TORCH_CHECK(state.dim() == 2 && state.size(1) == W);
+  check_groups(seq_cu, seq_slots, positions, T);
+  TORCH_CHECK(positions.numel() == T);
+  (void)max_rows;
+  const int S = seq_slots.numel();
+  DISPATCH_ACT(y_lin, fi::launch_rglru_scan<A>(
+                          ptr<A>(out), u.data_ptr<float>(),
+                          gate_lin.data_ptr<float>(),
+                          gate_bias.data_ptr<float>(), lam.data_ptr<float>(),
+                          ptr<A>(y_lin), y_lin.stride(0),
+                          state.data_ptr<float>(), seq_cu.data_ptr<int>(),
+                          seq_slots.data_ptr<int>(),
+                          positions.data_ptr<int>(), (int)T, S, (int)W,
+                          (int)(W / B), (float)decay_scale, stream()));
+}
+
+void relu_squared(at::Tensor out, at::Tensor x) {
+  CHECK_ACT(x);
+  CHECK_ACT(out);
+  TORCH_CHECK(x.dim() == 2 && out.is_contiguous() &&
+              out.sizes() == x.sizes() &&
+              out.scalar_type() == x.scalar_type());
+  check_rows(x, x.size(0), x.size(1), "relu input");
+  DISPATCH_ACT(x, fi::launch_relu_squared<A>(ptr<A>(out), ptr<A>(x),
+                                             x.stride(0), (int)x.size(0),
+                                             (int)x.size(1), stream()));
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("scaled_residual_layer_norm", &scaled_residual_layer_norm,
+        "fp32 stream += scaled sublayer results, then layer norm");
+  m.def("headnorm_qtemp_cache", &headnorm_qtemp_cache,
+        "weighted head RMS norms, query temperature, paged cache write");
+  m.def("latent_rope_cache", &latent_rope_cache,
+        "rotated query tails, normed latent + rotated key part to the cache");
+  m.def("sink_attention_splits", &sink_attention_splits,
+        "key spans of the split attention form for a cache capacity");
+  m.def("sink_attention_has_tiles", &sink_attention_has_tiles,
+        "whether the tiled attention form covers (key size, value size)");
+  m.def("sink_paged_attention", &sink_paged_attention,
+        "causal paged attention with sink, value slice and output gate");
+  m.def("causal_conv_state", &causal_conv_state,
+        "per-channel causal convolution with the tail kept per sequence");
+  m.def("rglru_scan", &rglru_scan, "gated linear recurrence times gelu branch");
+  m.def("relu_squared", &relu_squared, "relu(x)^2");
   m.def("layer_norm", &layer_norm, "layer norm of an fp32 stream, no bias");
   m.def("gated_residual_layer_norm", &gated_residual_layer_norm,
         "fp32 residual += y * sigmoid(gate); optional next layer norm");

@@ -404,6 +404,9 @@ def latent_rope_cache_(q, ckr, positions, inv_freq, norm_w, eps: float,
                            rank, q_out)
 
 
+SPLIT_ROWS_PER_LAUNCH = 512  # rows per launch of the split attention form
+
+
 def sink_paged_attention(q, k_cache, v_cache, seq_bt, row_seq, positions,
                          scale: float, sink=None, value_dims: int = 0,
                          out_gate=None, seq_cu=None, tiles=None):
@@ -418,16 +421,20 @@ def sink_paged_attention(q, k_cache, v_cache, seq_bt, row_seq, positions,
         out = torch.empty((T, H, V), dtype=q.dtype, device=q.device)
         tile_seq = tile_row0 = None
         tile_rows = 0
-        if tiles is not None and seq_cu is not None and tiles[2] > 0:
+        if (tiles is not None and seq_cu is not None and tiles[2] > 0
+                and _native().sink_attention_has_tiles(q.shape[2], V)):
             tile_seq, tile_row0, tile_rows = tiles
         rest = T - tile_rows
         part_ml = part_o = None
         if rest > 0:
+            # rows outside the tile table: partial results per span of the
+            # cache capacity, at most SPLIT_ROWS_PER_LAUNCH rows at a time
             bs = k_cache.shape[2]
             ns = _native().sink_attention_splits(seq_bt.shape[1] * bs)
-            part_ml = torch.empty((rest, H, ns, 2), dtype=torch.float32,
+            cap = min(rest, SPLIT_ROWS_PER_LAUNCH)
+            part_ml = torch.empty((cap, H, ns, 2), dtype=torch.float32,
                                   device=q.device)
-            part_o = torch.empty((rest, H, ns, V), dtype=torch.float32,
+            part_o = torch.empty((cap, H, ns, V), dtype=torch.float32,
                                  device=q.device)
         _native().sink_paged_attention(out, q, k_cache, v_cache, seq_bt,
                                        row_seq, positions, float(scale),
