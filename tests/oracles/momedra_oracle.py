@@ -55,6 +55,18 @@ def rotate_pairs(x, pos, dims, base):
     return y
 
 
+def attend(q, K, V, scale, sink=None):
+    """One query over the keys K [n, d] and values V [n, v]: softmax of
+    (K q) * scale, with exp(sink) added to the denominator when given."""
+    s = (K @ q) * scale
+    mx = s.max() if sink is None else torch.maximum(s.max(), sink)
+    e = torch.exp(s - mx)
+    den = e.sum()
+    if sink is not None:
+        den = den + torch.exp(sink - mx)
+    return ((e / den)[:, None] * V).sum(0)
+
+
 def gated_attention(h, P, pre, m, eps):
     """Grouped-query softmax attention without rotation: biased
     projections, weighted RMS norm of every query and key head, a query

@@ -1,0 +1,843 @@
+"""Momedra through the engine against the float64 oracle in
+tests/oracles/momedra_oracle.py: every mechanism alone, prompts against
+token-by-token decoding, portions down to two tokens, unequal batches,
+recycled pages and slots, far keys and span/tile/page borders, first
+tokens, long decoding, odd sizes, and greedy generation through the
+scheduler.
+
+The same cases run on the CPU ops (always) and on the HIP kernels (gpu
+marker)."""
+
+import copy
+import json
+import math
+import os
+
+import pytest
+import torch
+
+from fusioninfer_amd.config import CacheConfig, EngineConfig, SchedulerConfig
+from fusioninfer_amd.engine.llm_engine import LLMEngine
+from fusioninfer_amd.engine.metadata import AttnMetadata
+from fusioninfer_amd.engine.sequence import SamplingParams
+from fusioninfer_amd.models import registry
+from fusioninfer_amd.models.mixers import (
+    LatentAttention,
+    LatentAttentionConfig,
+    ParallelResidualLayer,
+    RGLRUConfig,
+    RGLRUMixer,
+    RoutedExperts,
+    TemperedGatedAttention,
+    TemperedGatedAttentionConfig,
+)
+from fusioninfer_amd.ops import seqmix
+from tests.oracles import momedra_oracle as oracle
+
+DEVICES = ["cpu", pytest.param("cuda", marks=pytest.mark.gpu)]
+F64 = torch.float64
+TOL = 2e-4   # fp32 engine vs float64 oracle, relative
+
+
+def dense_cfg(ff=40):
+    return {"kind": "dense", "ff": ff}
+
+
+def moe_cfg(ff=24, experts=5, top=2, shared=20):
+    m = {"kind": "moe", "expert": {"ff": ff},
+         "router": {"experts": experts, "top": top}}
+    if shared:
+        m["shared"] = {"ff": shared}
+    return m
+
+
+def attention_cfg(heads=4, kv_heads=2, dim=8, vdim=12, scale=0.3,
+                  coef=0.4, every=5, mlp=None):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+         "scale": scale}
+    if every:
+        m["q_temp"] = {"coef": coef, "every": every}
+    return {"type": "attention", "mixer": m, "mlp": mlp}
+
+
+def latent_cfg(heads=3, dim=8, rot_dim=6, vdim=10, rank=20, scale=0.25,
+               base=100.0, mlp=None):
+    return {"type": "latent_attention",
+            "mixer": {"heads": heads, "dim": dim, "rot_dim": rot_dim,
+                      "vdim": vdim, "kv_rank": rank, "scale": scale,
+                      "rot": {"base": base, "dims": rot_dim}},
+            "mlp": mlp}
+
+
+def rglru_cfg(width=36, blocks=3, conv=3, mlp=None):
+    return {"type": "rglru",
+            "mixer": {"width": width, "blocks": blocks, "conv": conv},
+            "mlp": mlp}
+
+
+def small_config():
+    """Sizes chosen so that nothing coincides: key, value, rotated and
+    latent sizes all differ, grouped heads, a temperature period that is
+    neither a power of two nor a multiple of the page size, layers that
+    differ, one layer without feed-forward, a repeated span of two layers
+    run three times with a layer before and after it."""
+    return {
+        "architecture": "Momedra",
+        "vocab": 89,
+        "width": 48,
+        "norm": {"eps": 1e-3},
+        "residual_mult": 0.7,
+        "loop": {"start": 1, "stop": 3, "times": 3},
+        "layers": [
+            rglru_cfg(mlp=moe_cfg()),
+            latent_cfg(mlp=dense_cfg()),
+            attention_cfg(mlp=None),
+            rglru_cfg(width=20, blocks=1, conv=4,
+                      mlp=moe_cfg(ff=16, experts=3, top=1, shared=0)),
+            attention_cfg(heads=6, kv_heads=1, dim=12, vdim=4, scale=0.11,
+                          coef=0.9, every=7, mlp=dense_cfg(24)),
+        ],
+    }
+
+
+def make_engine(raw, device, dtype="float32", blocks=64, max_seqs=4,
+                seed=0, budget=4096, eager=True):
+    mc = registry.model_config_from_dict(raw)
+    mc.dtype = dtype
+    cfg = EngineConfig(
+        model=mc,
+        cache=CacheConfig(num_gpu_blocks=blocks, enable_prefix_caching=False),
+        scheduler=SchedulerConfig(max_num_seqs=max_seqs,
+                                  max_num_batched_tokens=budget,
+                                  max_model_len=blocks * 16,
+                                  prefill_admission_tokens=0),
+        enforce_eager=eager,
+        num_state_slots=max_seqs,
+        seed=seed,
+    )
+    eng = LLMEngine(cfg, device=device)
+    model = eng.runner.model
+    # livelier weights than the 0.02-std init so that every branch matters
+    g = torch.Generator().manual_seed(seed + 2)
+    for name, p in model.named_parameters():
+        if p.dim() >= 2:
+            p.data.copy_((torch.randn(p.shape, generator=g)
+                          / math.sqrt(p.shape[-1])).to(p.dtype).to(p.device))
+    model.randomize_small_params(seed + 1)
+    for layer in model.layers:
+        if layer.routed is not None:
+            layer.routed.invalidate_packed()
+    W = {k: v.detach().cpu().to(F64)
+         for k, v in model.export_weights().items()}
+    return eng, W
+
+
+def rel_err(got, want):
+    """Mean-free RMS difference relative to the RMS of the expected row."""
+    got, want = got.double().cpu(), want.double().cpu()
+    d = got - want
+    d = d - d.mean(-1, keepdim=True)
+    w = want - want.mean(-1, keepdim=True)
+    return (d.pow(2).mean(-1).sqrt() / w.pow(2).mean(-1).sqrt()).max().item()
+
+
+def run_schedule(eng, steps):
+    """steps: [[(id, tokens, want)], ...] with ('end', id) tuples allowed;
+    returns {id: {position: logits}}."""
+    got, at = {}, {}
+    for step in steps:
+        entries = [e for e in step if e[0] != "end"]
+        end = [e[1] for e in step if e[0] == "end"]
+        out = eng.forced_step(entries, end).cpu()
+        row = 0
+        for rid, toks, want in entries:
+            for w in want:
+                got.setdefault(rid, {})[at.get(rid, 0) + w] = out[row]
+                row += 1
+            at[rid] = at.get(rid, 0) + len(toks)
+        for rid in end:
+            at.pop(rid, None)
+    return got
+
+
+def tokens(n, seed, vocab=89):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def mk(v, device):
+    return torch.tensor(v, dtype=torch.int32, device=device)
+
+
+def span_meta(spans, device, bs=16, pages=None, slots=None):
+    """Metadata of one step: spans = [(first position, rows)] of
+    different sequences; sequence s owns pages[s] (default: its own
+    consecutive run of 32 pages) and state slot slots[s]."""
+    pos, slot_map, row_seq, cu, bts = [], [], [], [0], []
+    for s, (p0, n) in enumerate(spans):
+        pg = pages[s] if pages else list(range(32 * s, 32 * s + 32))
+        bts.append(pg)
+        for r in range(n):
+            p = p0 + r
+            pos.append(p)
+            slot_map.append(pg[p // bs] * bs + p % bs)
+            row_seq.append(s)
+        cu.append(cu[-1] + n)
+    width = max(len(b) for b in bts)
+    bt = [b + [0] * (width - len(b)) for b in bts]
+    T = len(pos)
+    meta = AttnMetadata(num_prefill_tokens=T, num_decode_tokens=0,
+                        positions=mk(pos, device),
+                        slot_mapping=mk(slot_map, device))
+    meta.seq_cu = mk(cu, device)
+    meta.row_seq = mk(row_seq, device)
+    meta.seq_bt = mk(bt, device)
+    meta.seq_slots = mk(slots if slots is not None
+                        else list(range(len(spans))), device)
+    meta.max_seq_rows = max(n for _, n in spans)
+    lead = [n for _, n in spans if n > 1]
+    if lead and all(n > 1 for _, n in spans[: len(lead)]):
+        meta.seq_tiles = seqmix.build_attention_tiles(lead, device=device)
+    return meta
+
+
+def one_layer(mixer_cls, cfg, width, device, dtype=torch.float32, seed=0):
+    """A mixer behind the merged projection of a parallel-residual layer,
+    with lively weights, and its weights under the oracle's names."""
+    torch.manual_seed(seed)
+    mixer = mixer_cls(cfg, width, 1e-4, dtype)
+    layer = ParallelResidualLayer(mixer, None, None, width, 1e-4, 1.0, dtype)
+    g = torch.Generator().manual_seed(seed + 5)
+    for p in layer.parameters():
+        if p.dim() >= 2:
+            p.data.copy_((torch.randn(p.shape, generator=g)
+                          / math.sqrt(p.shape[-1])).to(p.dtype))
+    if layer.in_proj.bias is not None:
+        layer.in_proj.bias.data.copy_(
+            torch.randn(layer.in_proj.bias.shape, generator=g) * 0.2)
+        for br in layer.branches:
+            if br not in mixer.biased:
+                a, n = layer.in_proj_rows(br)
+                layer.in_proj.bias.data[a:a + n] = 0
+    P = {}
+    for br in mixer.in_names:
+        a, n = layer.in_proj_rows(br)
+        P[br] = layer.in_proj.weight.data[a:a + n].to(F64)
+        if layer.in_proj.bias is not None and br in mixer.biased:
+            P[br + ".b"] = layer.in_proj.bias.data[a:a + n].to(F64)
+    P["o"] = mixer.o_proj.weight.data.to(F64)
+    return layer.to(device), P, g
+
+
+def run_spans(layer, h, steps, device, caches):
+    """Feed rows of h (one sequence per entry of `steps[i]`) step by step;
+    steps: [[(seq, first position, rows)]]; h: {seq: [T, W]}."""
+    out = {s: torch.zeros(v.shape[0], layer.mixer.o_proj.weight.shape[0])
+           for s, v in h.items()}
+    for step in steps:
+        order = sorted(step, key=lambda e: e[2] == 1)   # portions first
+        meta = span_meta([(p0, n) for _, p0, n in order], device,
+                         pages=[list(range(32 * s, 32 * s + 32))
+                                for s, _, _ in order],
+                         slots=[s for s, _, _ in order])
+        x = torch.cat([h[s][p0:p0 + n] for s, p0, n in order]).to(device)
+        parts = layer.in_proj(x).split(layer.sizes, dim=-1)
+        y = layer.mixer(parts, meta, caches).cpu()
+        a = 0
+        for s, p0, n in order:
+            out[s][p0:p0 + n] = y[a:a + n]
+            a += n
+    return out
+
+
+MIXED_STEPS = [
+    [(0, 0, 2), (1, 0, 21)],
+    [(0, 2, 1), (1, 21, 2)],
+    [(0, 3, 17), (1, 23, 1)],
+    [(0, 20, 1), (1, 24, 1)],
+    [(0, 21, 19)],
+]
+
+
+# ------------------------------------------------------------ mechanisms
+@pytest.mark.parametrize("device", DEVICES)
+def test_scaled_residual_and_layer_norm(device):
+    torch.manual_seed(0)
+    W_, T = 44, 7
+    x = torch.randn(T, W_) * 3 + 1.5
+    w = torch.rand(W_) + 0.5
+    ys = [torch.randn(T, W_) for _ in range(3)]
+    for n in (1, 2, 3):
+        resid = x.clone().to(device)
+        h = seqmix.scaled_residual_layer_norm_(
+            resid, [y.to(device) for y in ys[:n]], [0.6] * n, w.to(device),
+            1e-3, torch.float32)
+        want_x = x.double() + 0.6 * sum(y.double() for y in ys[:n])
+        assert torch.allclose(resid.cpu().double(), want_x, atol=1e-5)
+        want_h = oracle.layer_norm(want_x, w.double(), 1e-3)
+        assert torch.allclose(h.cpu().double(), want_h, atol=1e-5)
+    resid = x.clone().to(device)
+    assert seqmix.scaled_residual_layer_norm_(
+        resid, [ys[0].to(device)], [1.0], None, 1e-3, torch.float32) is None
+    assert torch.allclose(resid.cpu(), x + ys[0], atol=1e-6)
+    r = seqmix.relu_squared((x - 1.5).to(device)).cpu()
+    assert torch.allclose(r, torch.relu(x - 1.5) ** 2, atol=1e-6)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("H,G,dim,vdim,coef,every", [
+    (4, 2, 8, 12, 0.4, 5), (6, 1, 12, 4, 0.9, 7), (3, 3, 10, 10, 0.0, 0),
+    (10, 1, 6, 5, 0.5, 1), (2, 2, 96, 96, 0.3, 16)])
+def test_gated_attention_matches_oracle(device, H, G, dim, vdim, coef,
+                                        every):
+    cfg = TemperedGatedAttentionConfig(H, G, dim, vdim, 0.21, coef, every)
+    layer, P, g = one_layer(TemperedGatedAttention, cfg, 40, device)
+    layer.mixer.q_norm.data.copy_(torch.rand(dim, generator=g) + 0.5)
+    layer.mixer.k_norm.data.copy_(torch.rand(dim, generator=g) + 0.5)
+    P["q.norm"] = layer.mixer.q_norm.data.cpu().to(F64)
+    P["k.norm"] = layer.mixer.k_norm.data.cpu().to(F64)
+    m = {"heads": H, "kv_heads": G, "dim": dim, "vdim": vdim, "scale": 0.21}
+    if every:
+        m["q_temp"] = {"coef": coef, "every": every}
+    h = {0: torch.randn(40, 40, generator=g),
+         1: torch.randn(25, 40, generator=g)}
+    caches = layer.mixer.state_tensors(64, 16, 2, device)
+    got = run_spans(layer, h, MIXED_STEPS, device, caches)
+    for s in h:
+        want = oracle.gated_attention(h[s].double(), P, "", m, 1e-4)
+        assert rel_err(got[s], want) < TOL, s
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("H,dim,rot,vdim,rank", [
+    (3, 8, 6, 10, 20), (1, 4, 2, 4, 7), (9, 6, 4, 5, 12), (2, 32, 16, 32, 96)])
+def test_latent_attention_matches_oracle(device, H, dim, rot, vdim, rank):
+    cfg = LatentAttentionConfig(H, dim, rot, vdim, rank, 0.27, 50.0)
+    layer, P, g = one_layer(LatentAttention, cfg, 40, device)
+    mx = layer.mixer
+    mx.c_norm.data.copy_(torch.rand(rank, generator=g) + 0.5)
+    mx.sink.data.copy_(torch.rand(H, generator=g) * 3 - 1)
+    P.update({"dkv.norm": mx.c_norm.data.cpu().to(F64),
+              "sink": mx.sink.data.cpu().to(F64),
+              "uk": mx.uk.data.cpu().to(F64), "uv": mx.uv.data.cpu().to(F64)})
+    m = {"heads": H, "dim": dim, "rot_dim": rot, "vdim": vdim,
+         "kv_rank": rank, "scale": 0.27, "rot": {"base": 50.0, "dims": rot}}
+    h = {0: torch.randn(40, 40, generator=g),
+         1: torch.randn(25, 40, generator=g)}
+    caches = mx.state_tensors(64, 16, 2, device)
+    got = run_spans(layer, h, MIXED_STEPS, device, caches)
+    for s in h:
+        want = oracle.latent_attention(h[s].double(), P, "", m, 1e-4)
+        assert rel_err(got[s], want) < TOL, s
+    # the sink matters: a large one takes most of the weight
+    mx.sink.data.fill_(9.0)
+    P["sink"] = mx.sink.data.cpu().to(F64)
+    got = run_spans(layer, {0: h[0]}, [[(0, 0, 40)]], device, caches)
+    want = oracle.latent_attention(h[0].double(), P, "", m, 1e-4)
+    assert rel_err(got[0], want) < TOL
+    assert got[0].abs().max() < 0.2 * want.abs().max() + 1.0
+
+
+def _crafted_attention(device, H, G, DK, DV, ctx, hot, alias, use_sink,
+                       use_gate, rows, dtype=torch.float32, seed=0):
+    """Keys/values straight in a paged cache with shuffled pages; the
+    query rows are aligned with the key at position `hot` so that its
+    score stands out; returns (got, want) for the last `rows` positions
+    run as one portion (rows > 1) or as a decoded row."""
+    g = torch.Generator().manual_seed(seed)
+    bs = 16
+    nblk = (ctx + bs - 1) // bs
+    perm = torch.randperm(nblk + 3, generator=g).tolist()[:nblk]
+    K = torch.randn(ctx, G, DK, generator=g)
+    V = K[:, :, :DV].clone() if alias else torch.randn(ctx, G, DV,
+                                                       generator=g)
+    q = torch.randn(rows, H, DK, generator=g) * 0.3
+    rep = H // G
+    for hh in range(H):
+        q[:, hh] += 3.0 * K[hot, hh // rep] / K[hot, hh // rep].norm()
+    K[hot] *= 4.0
+    if alias:
+        V = K[:, :, :DV].clone()
+    sink = (torch.rand(H, generator=g) * 2) if use_sink else None
+    gate = torch.randn(rows, H, generator=g) if use_gate else None
+    kc = torch.zeros(nblk + 3, G, bs, DK)
+    vc = None if alias else torch.zeros(nblk + 3, G, bs, DV)
+    for j in range(ctx):
+        kc[perm[j // bs], :, j % bs] = K[j]
+        if vc is not None:
+            vc[perm[j // bs], :, j % bs] = V[j]
+    p0 = ctx - rows
+    pos = list(range(p0, ctx))
+    tiles = (seqmix.build_attention_tiles([rows], device=device)
+             if rows > 1 else None)
+    out = seqmix.sink_paged_attention(
+        q.to(dtype).to(device), kc.to(dtype).to(device),
+        None if vc is None else vc.to(dtype).to(device),
+        mk([perm], device), mk([0] * rows, device), mk(pos, device), 0.5,
+        sink=None if sink is None else sink.to(device), value_dims=DV,
+        out_gate=None if gate is None else gate.to(dtype).to(device),
+        seq_cu=mk([0, rows], device), tiles=tiles)
+    want = torch.zeros(rows, H, DV, dtype=F64)
+    for r in range(rows):
+        for hh in range(H):
+            gg = hh // rep
+            o = oracle.attend(q[r, hh].double(), K[: pos[r] + 1, gg].double(),
+                              V[: pos[r] + 1, gg].double(), 0.5,
+                              None if sink is None else sink[hh].double())
+            if gate is not None:
+                o = o * oracle.sigmoid(gate[r, hh].double())
+            want[r, hh] = o
+    return out.float().cpu(), want
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("hot", [0, 15, 16, 63, 64, 127, 128, 255, 256, 298])
+@pytest.mark.parametrize("rows", [1, 2, 43])
+def test_far_key_at_page_span_and_tile_borders(device, hot, rows):
+    """One far key carries the weight; it sits at the borders of pages
+    (16), key tiles (64), row tiles (128) and key spans (256)."""
+    got, want = _crafted_attention(device, 4, 2, 96, 96, 300, hot,
+                                   alias=False, use_sink=False,
+                                   use_gate=True, rows=rows)
+    assert rel_err(got.reshape(rows, -1), want.reshape(rows, -1)) < TOL
+    got, want = _crafted_attention(device, 4, 1, 112, 96, 300, hot,
+                                   alias=True, use_sink=True, use_gate=False,
+                                   rows=rows, seed=1)
+    assert rel_err(got.reshape(rows, -1), want.reshape(rows, -1)) < TOL
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("H,G,DK,DV,alias", [
+    (3, 3, 7, 5, False), (12, 1, 22, 18, True), (16, 2, 64, 64, False),
+    (2, 1, 288, 256, True), (4, 4, 128, 128, False), (5, 1, 130, 260, False)])
+def test_attention_sizes_and_head_batches(device, H, G, DK, DV, alias):
+    for rows in (1, 140):
+        got, want = _crafted_attention(device, H, G, DK, DV, 270, 3, alias,
+                                       use_sink=True, use_gate=True,
+                                       rows=rows, seed=2)
+        assert rel_err(got.reshape(rows, -1), want.reshape(rows, -1)) < TOL
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("width,blocks,conv", [
+    (36, 3, 3), (20, 1, 4), (70, 2, 1), (130, 5, 2)])
+def test_rglru_conv_tail_and_state(device, width, blocks, conv):
+    cfg = RGLRUConfig(width, blocks, conv)
+    layer, P, g = one_layer(RGLRUMixer, cfg, 40, device)
+    mx = layer.mixer
+    mx.conv_w.data.copy_(torch.randn(width, conv, generator=g) * 0.5)
+    mx.conv_b.data.copy_(torch.randn(width, generator=g) * 0.1)
+    mx.gate_b.data.copy_(torch.randn(blocks, 2 * (width // blocks),
+                                     generator=g))
+    mx.lam.data.copy_(torch.rand(width, generator=g) * 4 - 3)
+    bw = width // blocks
+    P.update({"conv": mx.conv_w.data.cpu().to(F64),
+              "conv.b": mx.conv_b.data.cpu().to(F64),
+              "ra": mx.gate_w.data[:, :bw].cpu().to(F64),
+              "ri": mx.gate_w.data[:, bw:].cpu().to(F64),
+              "ra.b": mx.gate_b.data[:, :bw].cpu().to(F64),
+              "ri.b": mx.gate_b.data[:, bw:].cpu().to(F64),
+              "lam": mx.lam.data.cpu().to(F64)})
+    m = {"width": width, "blocks": blocks, "conv": conv}
+    h = {0: torch.randn(40, 40, generator=g),
+         1: torch.randn(25, 40, generator=g),
+         2: torch.randn(150, 40, generator=g)}
+    caches = mx.state_tensors(1, 16, 3, device)
+    # slots hold leftovers of earlier owners
+    for v in caches.values():
+        v.normal_()
+    steps = MIXED_STEPS + [[(2, 0, 131)], [(2, 131, 2)], [(2, 133, 1)],
+                           [(2, 134, 16)]]
+    got = run_spans(layer, h, steps, device, caches)
+    for s in h:
+        want = oracle.rglru_mixer(h[s].double(), P, "", m)
+        assert rel_err(got[s], want) < TOL, s
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_recurrence_keeps_a_far_token(device):
+    """Decays close to one: the first token's input still shows in the
+    state after two hundred rows, carried over many steps."""
+    cfg = RGLRUConfig(16, 1, 2)
+    layer, P, g = one_layer(RGLRUMixer, cfg, 24, device)
+    mx = layer.mixer
+    mx.lam.data.fill_(-9.0)          # softplus ~ 1e-4: a ~ 0.9996
+    mx.gate_b.data.fill_(2.0)
+    P.update({"conv": mx.conv_w.data.cpu().to(F64),
+              "conv.b": mx.conv_b.data.cpu().to(F64),
+              "ra": mx.gate_w.data[:, :16].cpu().to(F64),
+              "ri": mx.gate_w.data[:, 16:].cpu().to(F64),
+              "ra.b": mx.gate_b.data[:, :16].cpu().to(F64),
+              "ri.b": mx.gate_b.data[:, 16:].cpu().to(F64),
+              "lam": mx.lam.data.cpu().to(F64)})
+    h = torch.randn(200, 24, generator=g) * 0.05
+    h[0] *= 400.0
+    m = {"width": 16, "blocks": 1, "conv": 2}
+    want = oracle.rglru_mixer(h.double(), P, "", m)
+    h2 = h.clone()
+    h2[0] = 0
+    assert (want[-1] - oracle.rglru_mixer(h2.double(), P, "", m)[-1]
+            ).abs().max() > 0.1 * want[-1].abs().max()
+    caches = mx.state_tensors(1, 16, 1, device)
+    steps = [[(0, 0, 3)]] + [[(0, p, 1)] for p in range(3, 100)] + \
+        [[(0, 100, 98)], [(0, 198, 2)]]
+    got = run_spans(layer, {0: h}, steps, device, caches)
+    assert rel_err(got[0], want) < TOL
+
+
+def _experts_case(device, dtype, width, ff, E, top, T, seed=0):
+    torch.manual_seed(seed)
+    mod = RoutedExperts(width, ff, E, top, dtype, score="softmax",
+                        renorm=True, act="relu_sq", router_bias=True)
+    g = torch.Generator().manual_seed(seed + 1)
+    mod.gate_up.data.copy_((torch.randn(mod.gate_up.shape, generator=g)
+                            / math.sqrt(width)).to(dtype))
+    mod.down.data.copy_((torch.randn(mod.down.shape, generator=g)
+                         / math.sqrt(ff)).to(dtype))
+    mod.router.data.copy_(torch.randn(E, width, generator=g) * 0.3)
+    mod.router_bias.data.copy_(torch.randn(E, generator=g))
+    x = torch.randn(T, width, generator=g).to(dtype)
+    P = {"router": mod.router.data.to(F64),
+         "router.b": mod.router_bias.data.to(F64)}
+    for e in range(E):
+        P[f"e{e}.up"] = mod.gate_up.data[e].to(F64)
+        P[f"e{e}.down"] = mod.down.data[e].to(F64)
+    want = oracle.moe_ff(x.to(F64), P, "",
+                         {"router": {"experts": E, "top": top}})
+    mod = mod.to(device)
+    got = mod(x.to(device))
+    return got.float().cpu(), want
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("width,ff,E,top,T", [
+    (24, 10, 5, 2, 9), (16, 8, 1, 1, 3), (40, 12, 7, 7, 33), (64, 64, 3, 1, 1)])
+def test_squared_relu_experts_fp32(device, width, ff, E, top, T):
+    got, want = _experts_case(device, torch.float32, width, ff, E, top, T)
+    assert rel_err(got, want) < TOL
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("width,ff,E,top,T", [
+    (128, 64, 4, 2, 5), (256, 128, 8, 3, 300), (256, 64, 16, 4, 2100),
+    (96, 24, 5, 2, 17)])
+def test_squared_relu_experts_bf16_gpu(width, ff, E, top, T):
+    """Packed MFMA grouped GEMM where the sizes fit its tiles (both block
+    heights), the plain grouped kernel otherwise."""
+    got, want = _experts_case("cuda", torch.bfloat16, width, ff, E, top, T)
+    assert rel_err(got, want) < 3e-2
+
+
+# ----------------------------------------------------- model through engine
+@pytest.fixture(scope="module", params=DEVICES)
+def small(request):
+    raw = small_config()
+    eng, W = make_engine(raw, request.param)
+    toks = tokens(70, 11)
+    want = oracle.forward(toks, W, raw)
+    return raw, eng, W, toks, want
+
+
+def test_whole_prompt_layers_and_first_tokens(small):
+    raw, eng, W, toks, want = small
+    model = eng.runner.model
+    model.residual_trace = []
+    got = run_schedule(eng, [[("a", toks, list(range(len(toks))))],
+                             [("end", "a")]])
+    trace, model.residual_trace = model.residual_trace, None
+    rows = torch.stack([got["a"][p] for p in range(len(toks))])
+    assert rel_err(rows, want) < TOL
+    assert rel_err(rows[:3], want[:3]) < TOL
+    _, layers = oracle.forward(toks, W, raw, return_layers=True)
+    assert len(trace) == layers.shape[0] == 1 + 3 * 2 + 2
+    for got_x, want_x in zip(trace, layers):
+        assert rel_err(got_x, want_x) < TOL
+    one = run_schedule(eng, [[("b", toks[:1], [0])], [("end", "b")]])
+    assert rel_err(one["b"][0][None], want[:1]) < TOL
+
+
+def test_prefill_against_token_by_token_decoding(small):
+    raw, eng, W, toks, want = small
+    steps = [[("d", toks[:1], [0])]]
+    steps += [[("d", [t], [0])] for t in toks[1:]]
+    steps.append([("end", "d")])
+    got = run_schedule(eng, steps)
+    rows = torch.stack([got["d"][p] for p in range(len(toks))])
+    assert rel_err(rows, want) < TOL
+
+
+@pytest.mark.parametrize("sizes", [[2] * 35, [3, 16, 1, 2, 31, 2, 15],
+                                   [33, 2, 35], [64, 2, 2, 2]])
+def test_portions_of_several_sizes(small, sizes):
+    raw, eng, W, toks, want = small
+    assert sum(sizes) == len(toks)
+    steps, a = [], 0
+    for n in sizes:
+        steps.append([("p", toks[a:a + n], list(range(n)))])
+        a += n
+    steps.append([("end", "p")])
+    got = run_schedule(eng, steps)
+    rows = torch.stack([got["p"][p] for p in range(len(toks))])
+    assert rel_err(rows, want) < TOL
+
+
+def test_unequal_batch_equals_each_alone_and_recycles(small):
+    raw, eng, W, toks, want = small
+    reqs = {"r0": tokens(41, 1), "r1": tokens(5, 2), "r2": tokens(23, 3),
+            "r3": tokens(1, 4), "r4": tokens(37, 5), "r5": tokens(18, 6)}
+    ref = {k: oracle.forward(v, W, raw) for k, v in reqs.items()}
+    all_ = lambda n: list(range(n))
+    t = reqs
+    steps = [
+        [("r0", t["r0"][:7], all_(7)), ("r1", t["r1"][:2], all_(2))],
+        [("r0", t["r0"][7:8], [0]), ("r1", t["r1"][2:], all_(3)),
+         ("r2", t["r2"][:20], all_(20)), ("r3", t["r3"], [0]),
+         ("end", "r1"), ("end", "r3")],
+        # r4 and r5 take the slots and pages r1 and r3 gave back
+        [("r4", t["r4"][:30], all_(30)), ("r0", t["r0"][8:9], [0]),
+         ("r5", t["r5"][:1], [0]), ("r2", t["r2"][20:21], [0])],
+        [("r5", t["r5"][1:2], [0]), ("r0", t["r0"][9:41], all_(32)),
+         ("r2", t["r2"][21:], all_(2)), ("r4", t["r4"][30:31], [0]),
+         ("end", "r0"), ("end", "r2")],
+        [("r4", t["r4"][31:], all_(6)), ("r5", t["r5"][2:], all_(16)),
+         ("end", "r4"), ("end", "r5")],
+    ]
+    free_before = (eng.block_manager.num_free(), eng.state_manager.num_free())
+    got = run_schedule(eng, steps)
+    for k, v in reqs.items():
+        rows = torch.stack([got[k][p] for p in range(len(v))])
+        assert rel_err(rows, ref[k]) < TOL, k
+    assert (eng.block_manager.num_free(),
+            eng.state_manager.num_free()) == free_before
+
+
+def test_slot_and_pages_reused_by_a_shorter_request(small):
+    """A long request leaves state, a convolution tail and pages behind;
+    the next one in the same slot and pages must start from nothing."""
+    raw, eng, W, toks, want = small
+    run_schedule(eng, [[("x", tokens(60, 9), [])], [("end", "x")]])
+    got = run_schedule(eng, [[("y", toks[:2], [0, 1])],
+                             [("y", toks[2:9], list(range(7)))],
+                             [("end", "y")]])
+    rows = torch.stack([got["y"][p] for p in range(9)])
+    assert rel_err(rows, want[:9]) < TOL
+
+
+def test_greedy_generation_through_scheduler(small):
+    raw, eng, W, toks, want = small
+    prompts = [toks[:13], toks[20:23], toks[30:51]]
+    n_new = 12
+    outs = eng.generate(prompts, SamplingParams(max_tokens=n_new))
+    for p, o in zip(prompts, outs):
+        assert o.output_token_ids == oracle.greedy(p, W, raw, n_new)
+    assert eng.state_manager.num_free() == eng.state_manager.num_slots
+
+
+def test_generation_with_small_token_budget_chunks_prompts():
+    """The scheduler's own chunked prefill (budget 8 tokens a step) and
+    more requests than slots."""
+    raw = small_config()
+    eng, W = make_engine(raw, "cpu", max_seqs=2, budget=8, seed=3)
+    prompts = [tokens(21, 31), tokens(9, 32), tokens(14, 33)]
+    outs = eng.generate(prompts, SamplingParams(max_tokens=6))
+    for p, o in zip(prompts, outs):
+        assert o.output_token_ids == oracle.greedy(p, W, raw, 6)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_long_decoding_past_pages_spans_and_temperature_steps(device):
+    raw = {
+        "architecture": "Momedra", "vocab": 50, "width": 32,
+        "norm": {"eps": 1e-5}, "residual_mult": 1.0,
+        "loop": {"start": 0, "stop": 2, "times": 2},
+        "layers": [
+            attention_cfg(heads=2, kv_heads=2, dim=16, vdim=16, scale=0.25,
+                          coef=0.3, every=64,
+                          mlp=moe_cfg(ff=16, experts=4, top=2, shared=8)),
+            latent_cfg(heads=2, dim=8, rot_dim=8, vdim=8, rank=16,
+                       mlp=dense_cfg(16)),
+            rglru_cfg(width=16, blocks=2, conv=4),
+        ],
+    }
+    eng, W = make_engine(raw, device, blocks=24)
+    toks = tokens(300, 21, vocab=50)
+    want = oracle.forward(toks, W, raw)
+    steps = [[("a", toks[:10], list(range(10)))]]
+    steps += [[("a", [t], [0])] for t in toks[10:]]
+    got = run_schedule(eng, steps)
+    rows = torch.stack([got["a"][p] for p in range(len(toks))])
+    assert rel_err(rows, want) < TOL
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_values_that_could_hide_faults(device):
+    """Single heads, one block, no convolution, one expert, all experts
+    chosen, unit multiplier, temperature period one, no temperature, no
+    shared expert, no feed-forward, a span run once, a span that is the
+    whole model, no span at all, a recurrent-only model."""
+    toks = tokens(20, 7, vocab=31)
+    base = {"architecture": "Momedra", "vocab": 31, "width": 16,
+            "norm": {"eps": 1e-6}}
+    variants = [
+        dict(base, residual_mult=1.0,
+             loop={"start": 0, "stop": 3, "times": 1},
+             layers=[
+                 attention_cfg(heads=1, kv_heads=1, dim=8, vdim=8, scale=1.0,
+                               coef=1.0, every=1,
+                               mlp=moe_cfg(ff=8, experts=1, top=1, shared=0)),
+                 latent_cfg(heads=1, dim=4, rot_dim=2, vdim=4, rank=4,
+                            scale=1.0, base=1.0),
+                 rglru_cfg(width=8, blocks=1, conv=1,
+                           mlp=moe_cfg(ff=4, experts=3, top=3, shared=4))]),
+        dict(base, layers=[rglru_cfg(width=16, blocks=4, conv=2,
+                                     mlp=dense_cfg(8))]),
+        dict(base, residual_mult=0.25,
+             loop={"start": 0, "stop": 2, "times": 4},
+             layers=[attention_cfg(every=0, mlp=dense_cfg(8)),
+                     latent_cfg()]),
+    ]
+    for raw in variants:
+        eng, W = make_engine(raw, device, blocks=8)
+        want = oracle.forward(toks, W, raw)
+        got = run_schedule(eng, [[("a", toks[:11], list(range(11)))],
+                                 [("a", toks[11:13], [0, 1])],
+                                 [("a", toks[13:14], [0])],
+                                 [("a", toks[14:], list(range(6)))],
+                                 [("end", "a")]])
+        rows = torch.stack([got["a"][p] for p in range(len(toks))])
+        assert rel_err(rows, want) < TOL
+
+
+def test_checkpoint_directory_roundtrip(tmp_path):
+    """config.json + model.safetensors -> registry -> engine; bf16
+    storage; a checkpoint that lacks tensors is refused."""
+    from safetensors.torch import save_file
+
+    raw = small_config()
+    eng, W = make_engine(raw, "cpu", dtype="bfloat16")
+    disk = {k: v.to(torch.bfloat16) for k, v in
+            eng.runner.model.export_weights().items()}
+    d = tmp_path / "m"
+    os.makedirs(d)
+    save_file(disk, str(d / "model.safetensors"))
+    (d / "config.json").write_text(json.dumps(raw))
+    mc = registry.get_model_config(str(d))
+    assert mc.architecture == "Momedra"
+    assert registry.required_extensions(mc) == ("seqmix", "moe")
+    mc.dtype = "float32"
+    cfg = EngineConfig(model=mc, cache=CacheConfig(num_gpu_blocks=16),
+                       scheduler=SchedulerConfig(max_num_seqs=2,
+                                                 max_model_len=256),
+                       enforce_eager=True)
+    eng2 = LLMEngine(cfg, device="cpu")
+    W2 = {k: v.to(F64) for k, v in disk.items()}
+    toks = tokens(25, 8)
+    want = oracle.forward(toks, W2, raw)
+    got = run_schedule(eng2, [[("a", toks, list(range(25)))]])
+    rows = torch.stack([got["a"][p] for p in range(25)])
+    assert rel_err(rows, want) < TOL
+    with pytest.raises(ValueError):
+        eng2.runner.model.load_weights([("embed", disk["embed"])])
+    bad = copy.deepcopy(raw)
+    bad["layers"][0]["type"] = "unknown"
+    with pytest.raises(ValueError):
+        registry.model_config_from_dict(bad)
+    bad = copy.deepcopy(raw)
+    bad["loop"]["stop"] = 9
+    with pytest.raises(ValueError):
+        registry.model_config_from_dict(bad)
+
+
+def test_bf16_mode_stays_close_to_oracle():
+    raw = small_config()
+    eng, W = make_engine(raw, "cpu", dtype="bfloat16")
+    toks = tokens(40, 12)
+    want = oracle.forward(toks, W, raw)
+    got = run_schedule(eng, [[("a", toks[:30], list(range(30)))],
+                             [("a", toks[30:], list(range(10)))]])
+    rows = torch.stack([got["a"][p] for p in range(40)])
+    assert rel_err(rows, want) < 0.08
+
+
+def tiled_config():
+    """Sizes the tiled attention forms and the packed expert GEMM are
+    built for."""
+    return {
+        "architecture": "Momedra", "vocab": 211, "width": 256,
+        "norm": {"eps": 1e-5}, "residual_mult": 0.5,
+        "loop": {"start": 1, "stop": 3, "times": 2},
+        "layers": [
+            attention_cfg(heads=4, kv_heads=2, dim=128, vdim=128,
+                          scale=0.09, coef=0.3, every=64,
+                          mlp=dense_cfg(256)),
+            latent_cfg(heads=4, dim=32, rot_dim=16, vdim=32, rank=96,
+                       scale=0.14, base=250000.0,
+                       mlp=moe_cfg(ff=64, experts=8, top=2, shared=128)),
+            rglru_cfg(width=192, blocks=3, conv=4, mlp=dense_cfg(128)),
+            attention_cfg(heads=4, kv_heads=1, dim=64, vdim=64, scale=0.12,
+                          coef=0.2, every=32,
+                          mlp=moe_cfg(ff=128, experts=4, top=4, shared=64)),
+        ],
+    }
+
+
+@pytest.mark.gpu
+def test_hipgraph_decode_replays_match_oracle():
+    """All-decode steps replay captured graphs; replays interleave with
+    eager prompt steps and are checked every time."""
+    raw = small_config()
+    eng, W = make_engine(raw, "cuda", eager=False, max_seqs=4)
+    eng.runner.capture_decode_graphs()
+    reqs = {"a": tokens(30, 41), "b": tokens(22, 42), "c": tokens(17, 43)}
+    ref = {k: oracle.forward(v, W, raw) for k, v in reqs.items()}
+    steps = [[("a", reqs["a"][:9], list(range(9))),
+              ("b", reqs["b"][:4], list(range(4)))]]
+    for i in range(8):
+        steps.append([("a", [reqs["a"][9 + i]], [0]),
+                      ("b", [reqs["b"][4 + i]], [0])])
+    steps.append([("c", reqs["c"][:5], list(range(5))),
+                  ("a", [reqs["a"][17]], [0])])
+    for i in range(12):
+        steps.append([("a", [reqs["a"][18 + i]], [0]),
+                      ("b", [reqs["b"][12 + i // 2]], [0])] if i % 2 == 0
+                     else [("a", [reqs["a"][18 + i]], [0]),
+                           ("c", [reqs["c"][5 + i // 2]], [0])])
+    got = run_schedule(eng, steps)
+    for k in reqs:
+        for p, row in got[k].items():
+            assert rel_err(row[None], ref[k][p][None]) < TOL, (k, p)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_gpu_engine_matches_oracle_at_tiled_sizes(dtype):
+    raw = tiled_config()
+    eng, W = make_engine(raw, "cuda", dtype=dtype, blocks=40)
+    toks = tokens(330, 5, vocab=211)
+    want = oracle.forward(toks, W, raw)
+    got = run_schedule(eng, [[("a", toks[:200], list(range(200)))],
+                             [("a", toks[200:201], [0])],
+                             [("a", toks[201:329], list(range(128)))],
+                             [("a", toks[329:], [0])]])
+    rows = torch.stack([got["a"][p] for p in range(len(toks))])
+    if dtype == "float32":
+        assert rel_err(rows, want) < TOL
+        return
+    # bf16 rounds the router's input: at single positions a near-tie falls
+    # the other way and that row differs by an expert, so the bound is on
+    # the typical row and on how many rows stray
+    errs = torch.tensor([rel_err(rows[i:i + 1], want[i:i + 1])
+                         for i in range(len(toks))])
+    assert errs.median() < 0.03
+    assert (errs > 0.08).sum() <= 0.03 * len(toks)
+
+
+@pytest.mark.gpu
+def test_generation_with_graph_replay_and_pipelined_decode():
+    raw = small_config()
+    eng, W = make_engine(raw, "cuda", eager=False, max_seqs=4)
+    eng.runner.capture_decode_graphs()
+    prompts = [tokens(13, 51), tokens(3, 52), tokens(21, 53)]
+    outs = eng.generate(prompts, SamplingParams(max_tokens=10))
+    for p, o in zip(prompts, outs):
+        assert o.output_token_ids == oracle.greedy(p, W, raw, 10)
