@@ -72,14 +72,15 @@ def parse_args():
                         "workload mode; headline stays spec-off)")
     p.add_argument("--mixer-compare", action="store_true",
                    help="instead of the serving benchmark: prefill and "
-                        "decode token throughput of the Sefalorn and "
+                        "decode token throughput of the Momedra, Sefalorn and "
                         "Pinuvik designs at real-model layer sizes (random "
                         "weights) next to the Qwen3-style transformer of "
                         "the same sizes")
     p.add_argument("--mc-sizes", default="2048x16,4096x32",
                    help="WIDTHxHEADS list for --mixer-compare (head dim "
                         "128, kv heads = heads/4, ff = 3*width)")
-    p.add_argument("--mc-archs", default="sefalorn,pinuvik,transformer")
+    p.add_argument("--mc-archs",
+                   default="momedra,sefalorn,pinuvik,transformer")
     p.add_argument("--mc-layers", type=int, default=4)
     p.add_argument("--mc-prompt", type=int, default=2048)
     p.add_argument("--mc-prefill-seqs", type=int, default=4)
@@ -103,6 +104,41 @@ def _mixer_compare_config(arch, width, heads, layers, chunk, vocab=32000):
         mc.hidden_size, mc.num_layers = width, layers
         mc.num_heads, mc.num_kv_heads, mc.head_dim = heads, kv, dim
         mc.intermediate_size, mc.vocab_size = ff, vocab
+        return mc
+    if arch == "momedra":
+        # gated attention, latent attention (run twice as a repeated span)
+        # and the gated recurrence in turn; dense and routed feed-forwards
+        # alternate, the routed ones' active size (shared + top * ff)
+        # equals the dense ff
+        moe = {"kind": "moe", "expert": {"ff": ff // 4},
+               "router": {"experts": 8, "top": 2},
+               "shared": {"ff": ff // 2}}
+        dense = {"kind": "dense", "ff": ff}
+        attention = {
+            "type": "attention",
+            "mixer": {"heads": heads, "kv_heads": kv, "dim": dim,
+                      "vdim": dim, "scale": dim ** -0.5,
+                      "q_temp": {"coef": 0.1, "every": 1024}},
+            "mlp": dense}
+        latent = {
+            "type": "latent_attention",
+            "mixer": {"heads": heads, "dim": 96, "rot_dim": 32, "vdim": dim,
+                      "kv_rank": 256, "scale": dim ** -0.5,
+                      "rot": {"base": 1e6, "dims": 32}},
+            "mlp": moe}
+        rglru = {
+            "type": "rglru",
+            "mixer": {"width": width, "blocks": heads, "conv": 4},
+            "mlp": dense}
+        unit = [attention, latent, rglru]
+        n_layers = max(layers - 1, 1)
+        raw = {"architecture": "Momedra", "vocab": vocab, "width": width,
+               "norm": {"eps": 1e-5}, "residual_mult": 0.5,
+               "layers": [unit[i % 3] for i in range(n_layers)]}
+        if n_layers >= 2:
+            raw["loop"] = {"start": 1, "stop": 2, "times": 2}
+        mc = model_config_from_dict(raw)
+        mc.name = f"momedra-{width}x{heads}"
         return mc
     if arch == "sefalorn":
         # lightning and parallel layers in turn; the experts' active size

@@ -46,6 +46,16 @@ FI_DEV void ldv<u16, 4>(const u16* p, float* v) {
   for (int i = 0; i < 4; ++i) v[i] = bf16_to_f32(x.h[i]);
 }
 template <>
+FI_DEV void ldv<u16, 8>(const u16* p, float* v) {
+  const bf16x4 x = *reinterpret_cast<const bf16x4*>(p);
+  const bf16x4 y = *reinterpret_cast<const bf16x4*>(p + 4);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[i] = bf16_to_f32(x.h[i]);
+    v[4 + i] = bf16_to_f32(y.h[i]);
+  }
+}
+template <>
 FI_DEV void stv<float, 1>(float* p, const float* v) { *p = v[0]; }
 template <>
 FI_DEV void stv<u16, 1>(u16* p, const float* v) { *p = f32_to_bf16(v[0]); }

@@ -41,7 +41,7 @@ __global__ __launch_bounds__(256) void sink_attention_split_kernel(
     const int* __restrict__ seq_bt, int bt_stride,
     const int* __restrict__ row_seq, const int* __restrict__ positions,
     int row0, int H, int G, int DK, int DV, int dv_round, int bs, float scale,
-    int ns, int hb) {
+    int ns, int hb, int tpr) {
   extern __shared__ float smem[];
   float* qs = smem;                               // [kHeadBatch][DK]
   float* ps = qs + kHeadBatch * DK;               // [kHeadBatch][256]
@@ -122,6 +122,55 @@ __global__ __launch_bounds__(256) void sink_attention_split_kernel(
     ml[0] = m;
     ml[1] = l;
   }
+  if constexpr (VW > 1) {
+    if (tpr > 0) {
+      // vector form: tpr threads share a value row, VW columns each; the
+      // 64 / tpr key groups of a wave are folded by shuffles, the four
+      // waves through LDS (osum: [4][kHeadBatch][DV])
+      const int kgw = 64 / tpr;
+      const int dcol = (lane % tpr) * VW;
+      const int gid = wave * kgw + lane / tpr;
+      float acc[kHeadBatch][VW];
+#pragma unroll
+      for (int i = 0; i < kHeadBatch; ++i)
+#pragma unroll
+        for (int e = 0; e < VW; ++e) acc[i][e] = 0.f;
+      if (dcol < DV) {
+        for (int jj = gid; jj < nkeys; jj += 4 * kgw) {
+          float vv[VW];
+          ldv<A, VW>(v_cache + voff[jj] + dcol, vv);
+#pragma unroll
+          for (int i = 0; i < kHeadBatch; ++i) {
+            const float pj = ps[i * kSpanKeys + jj];
+#pragma unroll
+            for (int e = 0; e < VW; ++e) acc[i][e] += pj * vv[e];
+          }
+        }
+      }
+      for (int off = tpr; off < 64; off <<= 1)
+#pragma unroll
+        for (int i = 0; i < kHeadBatch; ++i)
+#pragma unroll
+          for (int e = 0; e < VW; ++e)
+            acc[i][e] += __shfl_xor(acc[i][e], off, 64);
+      if (lane < tpr && dcol < DV) {
+#pragma unroll
+        for (int i = 0; i < kHeadBatch; ++i)
+#pragma unroll
+          for (int e = 0; e < VW; ++e)
+            osum[(wave * kHeadBatch + i) * DV + dcol + e] = acc[i][e];
+      }
+      __syncthreads();
+      for (int idx = tid; idx < nh * DV; idx += 256) {
+        const int i = idx / DV, d = idx % DV;
+        part_o[((static_cast<int64_t>(r) * H + h0 + i) * ns + span) * DV + d] =
+            osum[i * DV + d] + osum[(kHeadBatch + i) * DV + d] +
+            osum[(2 * kHeadBatch + i) * DV + d] +
+            osum[(3 * kHeadBatch + i) * DV + d];
+      }
+      return;
+    }
+  }
   // weighted value sum: column d = tid % dv_round (+ dv_round ...), keys
   // dealt round-robin to the 256 / dv_round thread groups
   const int groups = max(1, 256 / dv_round);
@@ -193,7 +242,7 @@ typedef __attribute__((ext_vector_type(4))) short short4v;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 
-template <typename A, int DK, int DV, int BN, int QS>
+template <typename A, int DK, int DV, int BN, int QS, int HP>
 __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
     A* __restrict__ out, const A* __restrict__ q,
     const A* __restrict__ k_cache, const A* __restrict__ v_cache, int v_row,
@@ -210,14 +259,17 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
   constexpr int KB = DK / 16;
   constexpr int DB = DV / 16;
   constexpr int ROWS = 64 * QS;
+  // a wave keeps NQ query sets: QS row sets for each of HP heads that
+  // share the key/value head, so every K/V fragment read feeds NQ MFMAs
+  constexpr int NQ = QS * HP;
   __shared__ __attribute__((aligned(16))) A k_lds[BN * KP];
   __shared__ __attribute__((aligned(16))) A v_lds[BF ? DV * VP : BN * VP];
 
   const int tid = threadIdx.x;
   const int wave = tid / 64, lane = tid % 64;
   const int g4 = lane / 16, c16 = lane % 16;
-  const int h = blockIdx.y;
-  const int g = h / (H / G);
+  const int h0 = blockIdx.y * HP;
+  const int g = h0 / (H / G);
   const int s = tile_seq[blockIdx.x];
   // the tile table counts 128 rows per entry; with QS == 1 a workgroup
   // covers half an entry and blockIdx.z picks the half
@@ -231,17 +283,17 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
   const int p_first = positions[row_first];
   const int kv_hi = p_first + nrows - 1;   // positions in a group ascend by 1
 
-  int my_row[QS], my_pos[QS];
-  bool row_ok[QS];
-  short4v qf16[QS][BF ? KB : 1];
-  float qf32[QS][BF ? 1 : DK / 4];
+  int my_row[NQ], my_pos[NQ];
+  bool row_ok[NQ];
+  short4v qf16[NQ][BF ? KB : 1];
+  float qf32[NQ][BF ? 1 : DK / 4];
 #pragma unroll
-  for (int qs = 0; qs < QS; ++qs) {
-    my_row[qs] = (wave * QS + qs) * 16 + c16;
+  for (int qs = 0; qs < NQ; ++qs) {
+    my_row[qs] = (wave * QS + qs % QS) * 16 + c16;
     row_ok[qs] = my_row[qs] < nrows;
     my_pos[qs] = row_ok[qs] ? p_first + my_row[qs] : -1;
-    const A* qp =
-        q + (static_cast<int64_t>(row_first + my_row[qs]) * H + h) * DK;
+    const A* qp = q + (static_cast<int64_t>(row_first + my_row[qs]) * H +
+                       h0 + qs / QS) * DK;
     if constexpr (BF) {
 #pragma unroll
       for (int kk = 0; kk < KB; ++kk) {
@@ -258,10 +310,10 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
     }
   }
 
-  floatx4 o[QS][DB];
-  float m[QS], l[QS];
+  floatx4 o[NQ][DB];
+  float m[NQ], l[NQ];
 #pragma unroll
-  for (int qs = 0; qs < QS; ++qs) {
+  for (int qs = 0; qs < NQ; ++qs) {
     m[qs] = -INFINITY;
     l[qs] = 0.f;
 #pragma unroll
@@ -338,15 +390,15 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
 
     // ---- S^T = K Q^T ----
     const bool interior = wave_full && j0 + BN - 1 <= wave_min_pos;
-    float sv[QS][NB][4];
-    float tmax[QS];
+    float sv[NQ][NB][4];
+    float tmax[NQ];
 #pragma unroll
-    for (int qs = 0; qs < QS; ++qs) tmax[qs] = -INFINITY;
+    for (int qs = 0; qs < NQ; ++qs) tmax[qs] = -INFINITY;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
-      floatx4 acc[QS];
+      floatx4 acc[NQ];
 #pragma unroll
-      for (int qs = 0; qs < QS; ++qs) acc[qs] = floatx4{0.f, 0.f, 0.f, 0.f};
+      for (int qs = 0; qs < NQ; ++qs) acc[qs] = floatx4{0.f, 0.f, 0.f, 0.f};
       const A* kr = k_lds + (nb * 16 + c16) * KP;
       if constexpr (BF) {
 #pragma unroll
@@ -354,7 +406,7 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
           const short4v a =
               *reinterpret_cast<const short4v*>(kr + 16 * kk + 4 * g4);
 #pragma unroll
-          for (int qs = 0; qs < QS; ++qs)
+          for (int qs = 0; qs < NQ; ++qs)
             acc[qs] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
                 a, qf16[qs][kk], acc[qs], 0, 0, 0);
         }
@@ -363,13 +415,13 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
         for (int kk = 0; kk < DK / 4; ++kk) {
           const float a = kr[4 * kk + g4];
 #pragma unroll
-          for (int qs = 0; qs < QS; ++qs)
+          for (int qs = 0; qs < NQ; ++qs)
             acc[qs] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, qf32[qs][kk],
                                                            acc[qs], 0, 0, 0);
         }
       }
 #pragma unroll
-      for (int qs = 0; qs < QS; ++qs)
+      for (int qs = 0; qs < NQ; ++qs)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int key = j0 + nb * 16 + 4 * g4 + i;
@@ -379,7 +431,7 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
         }
     }
 #pragma unroll
-    for (int qs = 0; qs < QS; ++qs) {
+    for (int qs = 0; qs < NQ; ++qs) {
       float tm = tmax[qs];
       tm = fmaxf(tm, __shfl_xor(tm, 16, 64));
       tm = fmaxf(tm, __shfl_xor(tm, 32, 64));
@@ -406,9 +458,9 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
 
     // ---- O^T += V^T P^T ----
     if constexpr (BF) {
-      short4v pf[QS][NB];
+      short4v pf[NQ][NB];
 #pragma unroll
-      for (int qs = 0; qs < QS; ++qs)
+      for (int qs = 0; qs < NQ; ++qs)
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -422,7 +474,7 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
           const short4v a =
               *reinterpret_cast<const short4v*>(vr + nb * 16 + 4 * g4);
 #pragma unroll
-          for (int qs = 0; qs < QS; ++qs)
+          for (int qs = 0; qs < NQ; ++qs)
             o[qs][db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
                 a, pf[qs][nb], o[qs][db], 0, 0, 0);
         }
@@ -436,7 +488,7 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
           for (int i = 0; i < 4; ++i) {
             const float a = v_lds[(nb * 16 + 4 * g4 + i) * VP + db * 16 + c16];
 #pragma unroll
-            for (int qs = 0; qs < QS; ++qs)
+            for (int qs = 0; qs < NQ; ++qs)
               o[qs][db] = __builtin_amdgcn_mfma_f32_16x16x4f32(
                   a, sv[qs][nb][i], o[qs][db], 0, 0, 0);
           }
@@ -445,8 +497,9 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
   }
 
 #pragma unroll
-  for (int qs = 0; qs < QS; ++qs) {
+  for (int qs = 0; qs < NQ; ++qs) {
     if (!row_ok[qs]) continue;
+    const int h = h0 + qs / QS;
     float lt = l[qs];
     if (sink != nullptr) {
       // the sink joins the denominator in the domain of the running max
@@ -498,20 +551,23 @@ bool launch_sink_attention_tiles(A* out, const A* q, const A* k_cache,
                                  hipStream_t s) {
   constexpr bool BF = std::is_same<A, u16>::value;
   if (num_tiles == 0) return true;
-#define FI_TILE(K_, V_, BNB, BNF, QS_)                                         \
-  if (DK == K_ && DV == V_) {                                                  \
+  // head pairs (HP_ == 2) need an even number of heads per key/value head
+  const bool pairs = (H / G) % 2 == 0;
+#define FI_TILE(K_, V_, BNB, BNF, QS_, HP_)                                    \
+  if (DK == K_ && DV == V_ && (HP_ == 1 || pairs)) {                           \
     hipLaunchKernelGGL(                                                        \
-        (sink_attention_tile_kernel<A, K_, V_, (BF ? BNB : BNF), QS_>),        \
-        dim3(num_tiles, H, 2 / QS_), dim3(256), 0, s, out, q, k_cache,         \
+        (sink_attention_tile_kernel<A, K_, V_, (BF ? BNB : BNF), QS_, HP_>),   \
+        dim3(num_tiles, H / HP_, 2 / QS_), dim3(256), 0, s, out, q, k_cache,   \
         v_cache, v_row, seq_bt, bt_stride, seq_cu, positions, tile_seq,        \
         tile_row0, sink, gate, g_stride, H, G, block_size, scale);             \
     return true;                                                               \
   }
-  FI_TILE(64, 64, 64, 64, 2)
-  FI_TILE(96, 96, 64, 32, 2)
-  FI_TILE(128, 128, 64, 32, 2)
-  FI_TILE(112, 96, 64, 32, 2)
-  FI_TILE(288, 256, 32, 16, 1)
+  FI_TILE(64, 64, 64, 64, 2, 1)
+  FI_TILE(96, 96, 64, 32, 2, 1)
+  FI_TILE(128, 128, 64, 32, 2, 1)
+  FI_TILE(112, 96, 64, 32, 2, 1)
+  FI_TILE(288, 256, 32, 16, 1, 2)
+  FI_TILE(288, 256, 32, 16, 1, 1)
 #undef FI_TILE
   return false;   // caller falls back to the split form
 }
@@ -533,23 +589,42 @@ void launch_sink_attention_rows(A* out, float* part_ml, float* part_o,
   int dv_round = 1;
   while (dv_round < DV && dv_round < 256) dv_round *= 2;
   const int groups = max(1, 256 / dv_round);
+  constexpr bool BF = std::is_same<A, u16>::value;
+  // widest vector both the key rows and the value rows allow
+  int vw = 1;
+  if (BF && DK % 8 == 0) vw = 8;
+  else if (DK % 4 == 0) vw = 4;
+  // vector form of the value sum: whole vectors per value row, at most
+  // 64 threads a row, four partial copies within the LDS budget
+  int tpr = 0;
+  if (vw > 1 && DV % vw == 0 && v_row % vw == 0 && DV / vw <= 64 &&
+      DV <= 256) {
+    tpr = 1;
+    while (tpr < DV / vw) tpr *= 2;
+  }
+  const size_t osum_floats =
+      tpr > 0 ? static_cast<size_t>(4) * kHeadBatch * DV
+              : (groups > 1 ? static_cast<size_t>(groups) * kHeadBatch *
+                                  dv_round
+                            : 0);
   const size_t lds =
       (static_cast<size_t>(kHeadBatch) * DK + kHeadBatch * kSpanKeys +
-       2 * kHeadBatch * 4 +
-       (groups > 1 ? groups * kHeadBatch * dv_round : 0)) * sizeof(float);
+       2 * kHeadBatch * 4 + osum_floats) * sizeof(float);
   const dim3 grid(rows, G * nbg, ns);
-  constexpr bool BF = std::is_same<A, u16>::value;
-  const bool vec = DK % 4 == 0 && (BF || true);
-  if (vec)
-    hipLaunchKernelGGL((sink_attention_split_kernel<A, 4>), grid, dim3(256),
-                       lds, s, part_ml, part_o, q, k_cache, v_cache, v_row,
-                       seq_bt, bt_stride, row_seq, positions, row0, H, G, DK,
-                       DV, dv_round, block_size, scale, ns, hb);
-  else
-    hipLaunchKernelGGL((sink_attention_split_kernel<A, 1>), grid, dim3(256),
-                       lds, s, part_ml, part_o, q, k_cache, v_cache, v_row,
-                       seq_bt, bt_stride, row_seq, positions, row0, H, G, DK,
-                       DV, dv_round, block_size, scale, ns, hb);
+#define FI_SPLIT(VW_)                                                          \
+  hipLaunchKernelGGL((sink_attention_split_kernel<A, VW_>), grid, dim3(256),   \
+                     lds, s, part_ml, part_o, q, k_cache, v_cache, v_row,      \
+                     seq_bt, bt_stride, row_seq, positions, row0, H, G, DK,    \
+                     DV, dv_round, block_size, scale, ns, hb, tpr)
+  if constexpr (BF) {
+    if (vw == 8) FI_SPLIT(8);
+    else if (vw == 4) FI_SPLIT(4);
+    else FI_SPLIT(1);
+  } else {
+    if (vw == 4) FI_SPLIT(4);
+    else FI_SPLIT(1);
+  }
+#undef FI_SPLIT
   hipLaunchKernelGGL(sink_attention_combine_kernel<A>, dim3(rows, H), dim3(64),
                      0, s, out, part_ml, part_o, positions, sink, gate,
                      g_stride, row0, H, DV, ns);
