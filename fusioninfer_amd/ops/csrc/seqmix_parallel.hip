@@ -339,14 +339,20 @@ __global__ __launch_bounds__(64 * kScanWaves) void rglru_scan_kernel(
     state[static_cast<int64_t>(slot) * W + c] = carry;
 }
 
-template <typename A>
+template <typename A, int VW>
 __global__ __launch_bounds__(256) void relu_squared_kernel(
     A* __restrict__ out, const A* __restrict__ x, int64_t x_stride, int N) {
   const int64_t t = blockIdx.y;
-  const int i = blockIdx.x * 256 + threadIdx.x;
+  const int i = (blockIdx.x * 256 + threadIdx.x) * VW;
   if (i >= N) return;
-  const float v = fmaxf(Act<A>::ld(x + t * x_stride + i), 0.f);
-  Act<A>::st(out + t * N + i, v * v);
+  float v[VW];
+  ldv<A, VW>(x + t * x_stride + i, v);
+#pragma unroll
+  for (int e = 0; e < VW; ++e) {
+    v[e] = fmaxf(v[e], 0.f);
+    v[e] *= v[e];
+  }
+  stv<A, VW>(out + t * N + i, v);
 }
 
 }  // namespace
@@ -429,8 +435,17 @@ template <typename A>
 void launch_relu_squared(A* out, const A* x, int64_t x_stride, int T, int N,
                          hipStream_t st) {
   if (T == 0 || N == 0) return;
-  hipLaunchKernelGGL(relu_squared_kernel<A>, dim3(ceil_div(N, 256), T),
-                     dim3(256), 0, st, out, x, x_stride, N);
+  // four elements per thread when rows and the slice start allow it
+  const bool vec = N % 4 == 0 && x_stride % 4 == 0 &&
+                   reinterpret_cast<uintptr_t>(x) % (4 * sizeof(A)) == 0 &&
+                   reinterpret_cast<uintptr_t>(out) % (4 * sizeof(A)) == 0;
+  if (vec)
+    hipLaunchKernelGGL((relu_squared_kernel<A, 4>),
+                       dim3(ceil_div(N, 1024), T), dim3(256), 0, st, out, x,
+                       x_stride, N);
+  else
+    hipLaunchKernelGGL((relu_squared_kernel<A, 1>), dim3(ceil_div(N, 256), T),
+                       dim3(256), 0, st, out, x, x_stride, N);
 }
 
 #define FI_INST(A)                                                             \

@@ -254,7 +254,7 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
   constexpr bool BF = std::is_same<A, u16>::value;
   constexpr int VEC = BF ? 8 : 4;               // elements per 16-byte load
   constexpr int KP = DK + (BF ? 8 : 4);         // K tile [BN][KP]
-  constexpr int VP = BF ? BN + 8 : DV + 4;      // bf16: V^T [DV][VP]; fp32: V [BN][VP]
+  constexpr int VP = BF ? BN + 4 : DV + 4;      // bf16: V^T [DV][VP]; fp32: V [BN][VP]
   constexpr int NB = BN / 16;
   constexpr int KB = DK / 16;
   constexpr int DB = DV / 16;
@@ -349,8 +349,12 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
     if constexpr (BF) {
       // two adjacent keys per thread: the transposed V tile is written
       // with 4-byte stores (one (key, key+1) pair per d)
+      // lane quads take four adjacent key pairs of one column vector:
+      // their transposed stores fall into consecutive LDS words, and 16
+      // lanes still read 256 contiguous bytes of a key row
       for (int pid = tid; pid < (BN / 2) * VPR; pid += 256) {
-        const int kp = pid / VPR, dv = pid % VPR;
+        const int kp = (pid & 3) + 4 * (pid / (4 * VPR));
+        const int dv = (pid >> 2) % VPR;
         u32x4 v4[2];
 #pragma unroll
         for (int e2 = 0; e2 < 2; ++e2) {
