@@ -117,7 +117,7 @@ void launch_causal_conv_state(float*, const A*, int64_t, const float*,
 template <typename A>
 void launch_rglru_scan(A*, const float*, const float*, const float*,
                        const float*, const A*, int64_t, float*, const int*,
-                       const int*, const int*, int, int, int, int, float,
+                       const int*, const int*, int, int, int, int, float, int,
                        hipStream_t);
 template <typename A>
 void launch_relu_squared(A*, const A*, int64_t, int, int, hipStream_t);
@@ -1057,7 +1057,7 @@ void rglru_scan(at::Tensor out, at::Tensor u, at::Tensor gate_lin,
   TORCH_CHECK(state.dim() == 2 && state.size(1) == W);
   check_groups(seq_cu, seq_slots, positions, T);
   TORCH_CHECK(positions.numel() == T);
-  (void)max_rows;
+  TORCH_CHECK(max_rows >= 0);
   const int S = seq_slots.numel();
   DISPATCH_ACT(y_lin, fi::launch_rglru_scan<A>(
                           ptr<A>(out), u.data_ptr<float>(),
@@ -1067,7 +1067,8 @@ void rglru_scan(at::Tensor out, at::Tensor u, at::Tensor gate_lin,
                           state.data_ptr<float>(), seq_cu.data_ptr<int>(),
                           seq_slots.data_ptr<int>(),
                           positions.data_ptr<int>(), (int)T, S, (int)W,
-                          (int)(W / B), (float)decay_scale, stream()));
+                          (int)(W / B), (float)decay_scale, (int)max_rows,
+                          stream()));
 }
 
 void relu_squared(at::Tensor out, at::Tensor x) {

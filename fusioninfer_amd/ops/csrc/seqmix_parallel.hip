@@ -253,16 +253,17 @@ FI_DEV float softplus_f(float z) {
   return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z)));
 }
 
-constexpr int kScanWaves = 8;    // token chunks scanned side by side
-constexpr int kScanChunk = 8;    // tokens per wave and round
+constexpr int kScanWavesLong = 16;  // token chunks scanned side by side
+constexpr int kScanChunk = 8;       // tokens per wave and round
 
-// One workgroup: 64 channels (lanes) of one group, kScanWaves waves. A
+// One workgroup: 64 channels (lanes) of one group, kScanWaves waves (one
+// wave when no group of the step has more than a chunk of rows). A
 // round covers kScanWaves * kScanChunk consecutive rows: wave w scans its
 // chunk from a zero start keeping (product of decays, end value), the
 // waves exchange those through LDS, every wave derives the state at its
 // chunk's start from the carried state and the chunks before it, and
 // replays its chunk to write the outputs.
-template <typename A>
+template <typename A, int kScanWaves>
 __global__ __launch_bounds__(64 * kScanWaves) void rglru_scan_kernel(
     A* __restrict__ out,               // [T, W]
     const float* __restrict__ u,       // [T, W]
@@ -423,12 +424,20 @@ void launch_rglru_scan(A* out, const float* u, const float* gate_lin,
                        const A* y_lin, int64_t y_stride, float* state,
                        const int* seq_cu, const int* seq_slots,
                        const int* positions, int T, int S, int W, int bw,
-                       float decay_scale, hipStream_t st) {
+                       float decay_scale, int max_rows, hipStream_t st) {
   if (T == 0 || S == 0) return;
-  hipLaunchKernelGGL(rglru_scan_kernel<A>, dim3(S, ceil_div(W, 64)),
-                     dim3(64 * kScanWaves), 0, st, out, u, gate_lin,
-                     gate_bias, lam, y_lin, y_stride, state, seq_cu, seq_slots,
-                     positions, T, W, bw, decay_scale);
+  // max_rows: longest group of the step (0: unknown)
+  if (max_rows > 0 && max_rows <= kScanChunk)
+    hipLaunchKernelGGL((rglru_scan_kernel<A, 1>), dim3(S, ceil_div(W, 64)),
+                       dim3(64), 0, st, out, u, gate_lin, gate_bias, lam,
+                       y_lin, y_stride, state, seq_cu, seq_slots, positions, T,
+                       W, bw, decay_scale);
+  else
+    hipLaunchKernelGGL((rglru_scan_kernel<A, kScanWavesLong>),
+                       dim3(S, ceil_div(W, 64)), dim3(64 * kScanWavesLong), 0,
+                       st, out, u, gate_lin, gate_bias, lam, y_lin, y_stride,
+                       state, seq_cu, seq_slots, positions, T, W, bw,
+                       decay_scale);
 }
 
 template <typename A>
@@ -467,7 +476,7 @@ void launch_relu_squared(A* out, const A* x, int64_t x_stride, int T, int N,
   template void launch_rglru_scan<A>(                                          \
       A*, const float*, const float*, const float*, const float*, const A*,    \
       int64_t, float*, const int*, const int*, const int*, int, int, int, int, \
-      float, hipStream_t);                                                     \
+      float, int, hipStream_t);                                                   \
   template void launch_relu_squared<A>(A*, const A*, int64_t, int, int,        \
                                        hipStream_t);
 FI_INST(float)
