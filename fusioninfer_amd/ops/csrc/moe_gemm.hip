@@ -1,6 +1,6 @@
 // Grouped MFMA GEMM for MoE expert compute (gfx950).
 //
-// Replaces the round-1 capacity-padded torch.bmm experts (and their
+// Replaces capacity-padded torch.bmm experts (and their
 // per-layer `counts.max()` host sync) with a vLLM-style block-aligned
 // grouped GEMM: token assignments are sorted by expert and each expert's
 // segment is padded to a multiple of BLOCK_M on the DEVICE, so every
@@ -276,7 +276,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
 // quant) x B (e4m3, per-expert per-out-channel scales) on
 // mfma_f32_16x16x32_fp8_fp8 — HALF the weight bytes of bf16 in the
 // weight-bandwidth-bound decode regime, and no per-expert host loops:
-// the fp8 MoE path becomes hipGraph-capturable (round 1 ran per-expert
+// the fp8 MoE path becomes hipGraph-capturable (the first version ran per-expert
 // torch._scaled_mm with .nonzero() syncs). Same block-aligned layout
 // and epilogue structure as the bf16 kernel; dequant happens in the
 // epilogue: v = acc * a_scale[row] * b_scale[col].

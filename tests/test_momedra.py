@@ -748,6 +748,60 @@ def test_checkpoint_directory_roundtrip(tmp_path):
         registry.model_config_from_dict(bad)
 
 
+def test_schedule_replay_program(tmp_path):
+    """bin/trace_run on a checkpoint directory: steps on standard input,
+    one logits file per step that wants rows, a 'done' line per step, a
+    cache pool smaller than the sum of all requests."""
+    import subprocess
+    import sys
+
+    import numpy as np
+    from safetensors.torch import save_file
+
+    raw = small_config()
+    eng, W = make_engine(raw, "cpu", dtype="float32", seed=4)
+    d = tmp_path / "m"
+    os.makedirs(d)
+    save_file({k: v.to(torch.float32).contiguous() for k, v in
+               eng.runner.model.export_weights().items()},
+              str(d / "model.safetensors"))
+    (d / "config.json").write_text(json.dumps(raw))
+    a, b, c = tokens(70, 61), tokens(40, 62), tokens(50, 63)
+    steps = [
+        {"step": 0, "entries": [
+            {"id": "a", "tokens": a[:33], "want": [0, 32]},
+            {"id": "b", "tokens": b[:2], "want": []}], "end": []},
+        {"step": 1, "entries": [
+            {"id": "a", "tokens": a[33:34], "want": [0]},
+            {"id": "b", "tokens": b[2:], "want": [37]}], "end": ["b"]},
+        {"step": 2, "entries": [
+            {"id": "a", "tokens": a[34:], "want": []}], "end": ["a"]},
+        # c needs the pages a and b gave back
+        {"step": 3, "entries": [
+            {"id": "c", "tokens": c, "want": [49]}], "end": ["c"]},
+    ]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "out"
+    p = subprocess.run(
+        [sys.executable, os.path.join(root, "bin", "trace_run"), "--model",
+         str(d), "--dtype", "float32", "--out", str(out), "--max-tokens",
+         "128", "--device", "cpu"],
+        input="".join(json.dumps(s) + "\n" for s in steps), text=True,
+        capture_output=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    done = [ln for ln in p.stdout.splitlines() if ln.startswith("done ")]
+    assert done == ["done 0", "done 1", "done 2", "done 3"]
+    W64 = {k: v.to(F64) for k, v in W.items()}
+    wa, wb, wc = (oracle.forward(t, W64, raw) for t in (a, b, c))
+    V = raw["vocab"]
+    rd = lambda i: torch.from_numpy(
+        np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, V).copy())
+    assert rel_err(rd(0), wa[[0, 32]]) < TOL
+    assert rel_err(rd(1), torch.stack([wa[33], wb[39]])) < TOL
+    assert not (out / "2.f32").exists()
+    assert rel_err(rd(3), wc[49:50]) < TOL
+
+
 def test_bf16_mode_stays_close_to_oracle():
     raw = small_config()
     eng, W = make_engine(raw, "cpu", dtype="bfloat16")
