@@ -684,10 +684,16 @@ class LatentAttentionConfig:
     scale: float
     rot_base: float
     sink: bool = True        # learned per-head term in the denominator
+    rot_dims: int = -1       # leading entries of the rotated part that turn
+                             # (-1: all of it)
 
     def __post_init__(self):
-        if self.rot_dim % 2:
-            raise ValueError("rot_dim must be even")
+        if self.rot_dims < 0:
+            self.rot_dims = self.rot_dim
+        if self.rot_dim % 2 or self.rot_dims % 2:
+            raise ValueError("rot_dim and rot.dims must be even")
+        if self.rot_dims > self.rot_dim:
+            raise ValueError("rot.dims exceeds rot_dim")
 
 
 @dataclasses.dataclass
@@ -782,7 +788,7 @@ class LatentAttention(nn.Module):
         self.sink = _f32_param((H,), 0.0) if cfg.sink else None
         self.o_proj = RowParallelLinear(H * cfg.vdim, width, dtype=dtype)
         self.register_buffer(
-            "inv_freq", rotary_inv_freq(cfg.rot_dim, cfg.rot_base),
+            "inv_freq", rotary_inv_freq(cfg.rot_dims, cfg.rot_base),
             persistent=False)
 
     def state_tensors(self, num_blocks, block_size, num_slots, device):
@@ -807,8 +813,8 @@ class LatentAttention(nn.Module):
             cache["kv"], meta.slot_mapping, H, c.dim, c.rot_dim, c.rank, qf)
         # fold the key expansion into the queries: [H, T, dim] x [H, dim, rank]
         qu = q.view(T, H, c.dim + c.rot_dim)[:, :, : c.dim].transpose(0, 1)
-        qf[:, :, : c.rank] = torch.bmm(
-            qu, self.uk.view(H, c.dim, c.rank)).transpose(0, 1)
+        torch.bmm(qu, self.uk.view(H, c.dim, c.rank),
+                  out=qf.transpose(0, 1)[:, :, : c.rank])
         o = seqmix.sink_paged_attention(
             qf, cache["kv"], None, meta.seq_bt, meta.row_seq, meta.positions,
             c.scale, sink=self.sink, value_dims=c.rank, seq_cu=meta.seq_cu,

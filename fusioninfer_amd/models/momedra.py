@@ -128,14 +128,11 @@ def parse_config(raw: dict) -> MomedraConfig:
         elif kind == "latent_attention":
             rot = m.get("rot") or {}
             rot_dim = int(m["rot_dim"])
-            if int(rot.get("dims", rot_dim)) != rot_dim:
-                raise ValueError(
-                    f"layer {i}: the rotated part is rot_dim wide "
-                    f"(rot.dims {rot.get('dims')} != rot_dim {rot_dim})")
             mixer = LatentAttentionConfig(
                 heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=rot_dim,
                 vdim=int(m.get("vdim", m["dim"])), rank=int(m["kv_rank"]),
-                scale=float(m["scale"]), rot_base=float(rot["base"]))
+                scale=float(m["scale"]), rot_base=float(rot["base"]),
+                rot_dims=int(rot.get("dims", rot_dim)))
         elif kind == "rglru":
             mixer = RGLRUConfig(width=int(m["width"]),
                                 blocks=int(m.get("blocks", 1)),
@@ -405,6 +402,8 @@ class MomedraLM(nn.Module):
         if names is None:
             names = self._names = self._name_map()
         if name not in names:
+            if name == "loop.in" and self.loop_in is None:
+                return      # no repeated span configured: nothing enters it
             raise ValueError(f"unknown tensor {name!r}")
         param, spec = names[name]
         dst = self._view(param, spec)

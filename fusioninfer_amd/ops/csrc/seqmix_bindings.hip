@@ -108,7 +108,7 @@ template <typename A>
 void launch_latent_rope_cache(A*, const A*, int64_t, const A*, int64_t,
                               const int*, const float*, const float*, float,
                               A*, const int*, int, int, int, int, int, int,
-                              hipStream_t);
+                              int, hipStream_t);
 template <typename A>
 void launch_causal_conv_state(float*, const A*, int64_t, const float*,
                               const float*, float*, const int*, const int*,
@@ -872,7 +872,7 @@ void latent_rope_cache(at::Tensor q_out, at::Tensor q, at::Tensor ckr,
               q_out.size(0) == T && q_out.size(1) == H &&
               q_out.size(2) == C + R);
   TORCH_CHECK(positions.numel() == T && slot_mapping.numel() == T);
-  TORCH_CHECK(R % 2 == 0 && inv_freq.numel() == R / 2 && norm_w.numel() == C);
+  TORCH_CHECK(R % 2 == 0 && inv_freq.numel() <= R / 2 && norm_w.numel() == C);
   TORCH_CHECK(kv_cache.is_cuda() && kv_cache.is_contiguous() &&
               kv_cache.scalar_type() == dt && kv_cache.dim() == 4 &&
               kv_cache.size(1) == 1 && kv_cache.size(3) == C + R);
@@ -882,7 +882,8 @@ void latent_rope_cache(at::Tensor q_out, at::Tensor q, at::Tensor ckr,
                       inv_freq.data_ptr<float>(), norm_w.data_ptr<float>(),
                       (float)eps, ptr<A>(kv_cache),
                       slot_mapping.data_ptr<int>(), (int)T, (int)H, (int)D,
-                      (int)R, (int)C, (int)kv_cache.size(2), stream()));
+                      (int)R, (int)C, (int)inv_freq.numel(),
+                      (int)kv_cache.size(2), stream()));
 }
 
 int64_t sink_attention_splits(int64_t max_keys) {

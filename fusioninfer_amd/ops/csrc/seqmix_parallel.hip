@@ -142,7 +142,7 @@ __global__ __launch_bounds__(64) void latent_rope_cache_kernel(
     const int* __restrict__ positions, const float* __restrict__ inv_freq,
     const float* __restrict__ norm_w, float eps, A* __restrict__ kv_cache,
     const int* __restrict__ slot_mapping, int H, int D, int R, int C,
-    int bs) {
+    int rot_pairs, int bs) {
   const int t = blockIdx.x;
   const int hh = blockIdx.y;   // [0,H): query heads, H: the cache row
   const int lane = threadIdx.x;
@@ -170,7 +170,8 @@ __global__ __launch_bounds__(64) void latent_rope_cache_kernel(
     src = cs + C;
     dst = row + C;
   }
-  for (int i = lane; i < R / 2; i += 64) {
+  // the first rot_pairs pairs turn, the rest of the part passes
+  for (int i = lane; i < rot_pairs; i += 64) {
     const float u = Act<A>::ld(src + 2 * i);
     const float w = Act<A>::ld(src + 2 * i + 1);
     float sn, cs;
@@ -178,6 +179,7 @@ __global__ __launch_bounds__(64) void latent_rope_cache_kernel(
     Act<A>::st(dst + 2 * i, u * cs - w * sn);
     Act<A>::st(dst + 2 * i + 1, w * cs + u * sn);
   }
+  for (int d = 2 * rot_pairs + lane; d < R; d += 64) dst[d] = src[d];
 }
 
 constexpr int kMaxTaps = 16;
@@ -392,12 +394,13 @@ void launch_latent_rope_cache(A* q_out, const A* q, int64_t q_stride,
                               const int* positions, const float* inv_freq,
                               const float* norm_w, float eps, A* kv_cache,
                               const int* slot_mapping, int T, int H, int D,
-                              int R, int C, int bs, hipStream_t st) {
+                              int R, int C, int rot_pairs, int bs,
+                              hipStream_t st) {
   if (T == 0) return;
   hipLaunchKernelGGL(latent_rope_cache_kernel<A>, dim3(T, H + 1), dim3(64), 0,
                      st, q_out, q, q_stride, ckr, c_stride, positions,
                      inv_freq, norm_w, eps, kv_cache, slot_mapping, H, D, R, C,
-                     bs);
+                     rot_pairs, bs);
 }
 
 template <typename A>
@@ -467,7 +470,7 @@ void launch_relu_squared(A* out, const A* x, int64_t x_stride, int T, int N,
       int, int, int, int, int, hipStream_t);                                   \
   template void launch_latent_rope_cache<A>(                                   \
       A*, const A*, int64_t, const A*, int64_t, const int*, const float*,      \
-      const float*, float, A*, const int*, int, int, int, int, int, int,       \
+      const float*, float, A*, const int*, int, int, int, int, int, int, int,  \
       hipStream_t);                                                            \
   template void launch_causal_conv_state<A>(                                   \
       float*, const A*, int64_t, const float*, const float*, float*,           \

@@ -462,12 +462,14 @@ def headnorm_qtemp_cache_(q, k, v, positions, q_w, k_w, eps: float,
 
 
 def _rotate_interleaved(x, ang):
-    """Pairs (2i, 2i+1) of the last dim of x turned by ang[..., i]."""
+    """Pairs (2i, 2i+1) of the last dim of x turned by ang[..., i]; pairs
+    beyond the angles given pass unchanged."""
+    n = 2 * ang.shape[-1]
     cs, sn = torch.cos(ang), torch.sin(ang)
-    u, w = x[..., 0::2], x[..., 1::2]
-    out = torch.empty_like(x)
-    out[..., 0::2] = u * cs - w * sn
-    out[..., 1::2] = w * cs + u * sn
+    u, w = x[..., 0:n:2], x[..., 1:n:2]
+    out = x.clone()
+    out[..., 0:n:2] = u * cs - w * sn
+    out[..., 1:n:2] = w * cs + u * sn
     return out
 
 
@@ -475,7 +477,8 @@ def latent_rope_cache_(q, ckr, positions, inv_freq, norm_w, eps: float,
                        kv_cache, slot_mapping, num_heads: int, dim: int,
                        rot_dim: int, rank: int, q_out):
     """q [T, H*(dim+rot_dim)]: the trailing rot_dim entries of every head
-    are rotated (interleaved pairs, fp32 angle = position * inv_freq) and
+    are rotated (interleaved pairs, fp32 angle = position * inv_freq; pairs
+    beyond len(inv_freq) pass) and
     written to q_out[:, :, rank:]. ckr [T, rank+rot_dim]: the leading rank
     entries are RMS-normed with norm_w, the trailing rot_dim rotated; the
     row goes to kv_cache [B, 1, bs, rank+rot_dim] at slot_mapping."""

@@ -103,16 +103,18 @@ def latent_attention(h, P, pre, m, eps):
     H, D, R, V, C = m["heads"], m["dim"], m["rot_dim"], \
         m.get("vdim", m["dim"]), m["kv_rank"]
     base = m["rot"]["base"]
+    dims = m["rot"].get("dims", R)      # leading entries of the part that turn
     q = (h @ P[pre + "q"].T).view(T, H, D + R)
     ckr = h @ P[pre + "dkv"].T
     c = rms_norm(ckr[:, :C], P[pre + "dkv.norm"], eps)
-    kr = torch.stack([rotate_pairs(ckr[t, C:], t, R, base) for t in range(T)])
+    kr = torch.stack([rotate_pairs(ckr[t, C:], t, dims, base)
+                      for t in range(T)])
     ku = (c @ P[pre + "uk"].T).view(T, H, D)
     v = (c @ P[pre + "uv"].T).view(T, H, V)
     out = torch.zeros(T, H, V, dtype=F64)
     for t in range(T):
         for hh in range(H):
-            qr = rotate_pairs(q[t, hh, D:], t, R, base)
+            qr = rotate_pairs(q[t, hh, D:], t, dims, base)
             s = (ku[: t + 1, hh] @ q[t, hh, :D] + kr[: t + 1] @ qr) \
                 * m["scale"]
             e = torch.exp(s - s.max())

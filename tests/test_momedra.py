@@ -61,11 +61,12 @@ def attention_cfg(heads=4, kv_heads=2, dim=8, vdim=12, scale=0.3,
 
 
 def latent_cfg(heads=3, dim=8, rot_dim=6, vdim=10, rank=20, scale=0.25,
-               base=100.0, mlp=None):
+               base=100.0, mlp=None, dims=None):
     return {"type": "latent_attention",
             "mixer": {"heads": heads, "dim": dim, "rot_dim": rot_dim,
                       "vdim": vdim, "kv_rank": rank, "scale": scale,
-                      "rot": {"base": base, "dims": rot_dim}},
+                      "rot": {"base": base,
+                              "dims": rot_dim if dims is None else dims}},
             "mlp": mlp}
 
 
@@ -309,10 +310,13 @@ def test_gated_attention_matches_oracle(device, H, G, dim, vdim, coef,
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("H,dim,rot,vdim,rank", [
-    (3, 8, 6, 10, 20), (1, 4, 2, 4, 7), (9, 6, 4, 5, 12), (2, 32, 16, 32, 96)])
-def test_latent_attention_matches_oracle(device, H, dim, rot, vdim, rank):
-    cfg = LatentAttentionConfig(H, dim, rot, vdim, rank, 0.27, 50.0)
+@pytest.mark.parametrize("H,dim,rot,vdim,rank,dims", [
+    (3, 8, 6, 10, 20, 6), (1, 4, 2, 4, 7, 2), (9, 6, 4, 5, 12, 4),
+    (2, 32, 16, 32, 96, 16), (3, 8, 10, 6, 20, 4), (2, 8, 4, 8, 16, 0)])
+def test_latent_attention_matches_oracle(device, H, dim, rot, vdim, rank,
+                                         dims):
+    cfg = LatentAttentionConfig(H, dim, rot, vdim, rank, 0.27, 50.0,
+                                rot_dims=dims)
     layer, P, g = one_layer(LatentAttention, cfg, 40, device)
     mx = layer.mixer
     mx.c_norm.data.copy_(torch.rand(rank, generator=g) + 0.5)
@@ -321,7 +325,8 @@ def test_latent_attention_matches_oracle(device, H, dim, rot, vdim, rank):
               "sink": mx.sink.data.cpu().to(F64),
               "uk": mx.uk.data.cpu().to(F64), "uv": mx.uv.data.cpu().to(F64)})
     m = {"heads": H, "dim": dim, "rot_dim": rot, "vdim": vdim,
-         "kv_rank": rank, "scale": 0.27, "rot": {"base": 50.0, "dims": rot}}
+         "kv_rank": rank, "scale": 0.27,
+         "rot": {"base": 50.0, "dims": dims}}
     h = {0: torch.randn(40, 40, generator=g),
          1: torch.randn(25, 40, generator=g)}
     caches = mx.state_tensors(64, 16, 2, device)
@@ -685,8 +690,8 @@ def test_values_that_could_hide_faults(device):
                  attention_cfg(heads=1, kv_heads=1, dim=8, vdim=8, scale=1.0,
                                coef=1.0, every=1,
                                mlp=moe_cfg(ff=8, experts=1, top=1, shared=0)),
-                 latent_cfg(heads=1, dim=4, rot_dim=2, vdim=4, rank=4,
-                            scale=1.0, base=1.0),
+                 latent_cfg(heads=1, dim=4, rot_dim=4, vdim=4, rank=4,
+                            scale=1.0, base=1.0, dims=2),
                  rglru_cfg(width=8, blocks=1, conv=1,
                            mlp=moe_cfg(ff=4, experts=3, top=3, shared=4))]),
         dict(base, layers=[rglru_cfg(width=16, blocks=4, conv=2,
