@@ -330,67 +330,107 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
   const int wave_min_pos = wave_rows > 0 ? p_first + wave * 16 * QS : -1;
   const bool wave_full = wave_rows == 16 * QS;
 
-  for (int j0 = 0; j0 <= kv_hi; j0 += BN) {
-    // ---- stage K and V tiles (zero-filled past the range) ----
-    constexpr int KPR = DK / VEC;              // vectors per key row
-    constexpr int VPR = DV / VEC;
-    for (int vid = tid; vid < BN * KPR; vid += 256) {
-      const int key_l = vid / KPR, dv = vid % KPR;
-      const int key = j0 + key_l;
-      u32x4 kv4 = {0u, 0u, 0u, 0u};
-      if (key <= kv_hi) {
-        const int64_t rowi =
-            (static_cast<int64_t>(bt[key / block_size]) * G + g) * block_size +
-            key % block_size;
-        kv4 = *reinterpret_cast<const u32x4*>(k_cache + rowi * DK + dv * VEC);
-      }
-      *reinterpret_cast<u32x4*>(k_lds + key_l * KP + dv * VEC) = kv4;
+  // K and V tiles travel global -> registers -> LDS. With PF (the large
+  // sizes, whose register budget is spent anyway) the loads of the NEXT
+  // tile are issued right after the barrier that publishes the current
+  // one, so they are in flight during the MFMA phases; the small sizes
+  // load at the top of the iteration and keep the registers for a third
+  // wave per SIMD.
+  constexpr bool PF = QS == 1;
+  constexpr int KPR = DK / VEC;                // vectors per key row
+  constexpr int VPR = DV / VEC;
+  constexpr int KV = (BN * KPR + 255) / 256;   // K vectors per thread
+  constexpr int VN = BF ? ((BN / 2) * VPR + 255) / 256   // V key pairs
+                        : (BN * VPR + 255) / 256;        // V vectors
+  u32x4 kreg[KV];
+  u32x4 vreg[VN][BF ? 2 : 1];
+  auto row_index = [&](int key) {
+    return (static_cast<int64_t>(bt[key / block_size]) * G + g) * block_size +
+           key % block_size;
+  };
+  auto load_tile = [&](int j0) {
+#pragma unroll
+    for (int i = 0; i < KV; ++i) {
+      const int vid = tid + 256 * i;
+      const int key = j0 + vid / KPR;
+      kreg[i] = u32x4{0u, 0u, 0u, 0u};
+      if (vid < BN * KPR && key <= kv_hi)
+        kreg[i] = *reinterpret_cast<const u32x4*>(
+            k_cache + row_index(key) * DK + (vid % KPR) * VEC);
     }
     if constexpr (BF) {
-      // two adjacent keys per thread: the transposed V tile is written
-      // with 4-byte stores (one (key, key+1) pair per d)
       // lane quads take four adjacent key pairs of one column vector:
       // their transposed stores fall into consecutive LDS words, and 16
       // lanes still read 256 contiguous bytes of a key row
-      for (int pid = tid; pid < (BN / 2) * VPR; pid += 256) {
+#pragma unroll
+      for (int i = 0; i < VN; ++i) {
+        const int pid = tid + 256 * i;
         const int kp = (pid & 3) + 4 * (pid / (4 * VPR));
         const int dv = (pid >> 2) % VPR;
-        u32x4 v4[2];
 #pragma unroll
         for (int e2 = 0; e2 < 2; ++e2) {
           const int key = j0 + 2 * kp + e2;
-          v4[e2] = u32x4{0u, 0u, 0u, 0u};
-          if (key <= kv_hi) {
-            const int64_t rowi =
-                (static_cast<int64_t>(bt[key / block_size]) * G + g) *
-                    block_size + key % block_size;
-            v4[e2] = *reinterpret_cast<const u32x4*>(v_cache + rowi * v_row +
-                                                     dv * VEC);
-          }
+          vreg[i][e2] = u32x4{0u, 0u, 0u, 0u};
+          if (pid < (BN / 2) * VPR && key <= kv_hi)
+            vreg[i][e2] = *reinterpret_cast<const u32x4*>(
+                v_cache + row_index(key) * v_row + dv * VEC);
         }
-        const u16* va = reinterpret_cast<const u16*>(&v4[0]);
-        const u16* vb = reinterpret_cast<const u16*>(&v4[1]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < VN; ++i) {
+        const int vid = tid + 256 * i;
+        const int key = j0 + vid / VPR;
+        vreg[i][0] = u32x4{0u, 0u, 0u, 0u};
+        if (vid < BN * VPR && key <= kv_hi)
+          vreg[i][0] = *reinterpret_cast<const u32x4*>(
+              v_cache + row_index(key) * v_row + (vid % VPR) * VEC);
+      }
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int i = 0; i < KV; ++i) {
+      const int vid = tid + 256 * i;
+      if (vid < BN * KPR)
+        *reinterpret_cast<u32x4*>(k_lds + (vid / KPR) * KP +
+                                  (vid % KPR) * VEC) = kreg[i];
+    }
+    if constexpr (BF) {
+      // the transposed V tile is written with 4-byte stores: one
+      // (key, key+1) pair per value column
+#pragma unroll
+      for (int i = 0; i < VN; ++i) {
+        const int pid = tid + 256 * i;
+        if (pid >= (BN / 2) * VPR) continue;
+        const int kp = (pid & 3) + 4 * (pid / (4 * VPR));
+        const int dv = (pid >> 2) % VPR;
+        const u16* va = reinterpret_cast<const u16*>(&vreg[i][0]);
+        const u16* vb = reinterpret_cast<const u16*>(&vreg[i][1]);
 #pragma unroll
         for (int e = 0; e < 8; ++e)
           *reinterpret_cast<u32*>(v_lds + (dv * 8 + e) * VP + 2 * kp) =
               static_cast<u32>(va[e]) | (static_cast<u32>(vb[e]) << 16);
       }
     } else {
-      for (int vid = tid; vid < BN * VPR; vid += 256) {
-        const int key_l = vid / VPR, dv = vid % VPR;
-        const int key = j0 + key_l;
-        u32x4 vv4 = {0u, 0u, 0u, 0u};
-        if (key <= kv_hi) {
-          const int64_t rowi =
-              (static_cast<int64_t>(bt[key / block_size]) * G + g) *
-                  block_size + key % block_size;
-          vv4 = *reinterpret_cast<const u32x4*>(v_cache + rowi * v_row +
-                                                dv * VEC);
-        }
-        *reinterpret_cast<u32x4*>(v_lds + key_l * VP + dv * VEC) = vv4;
+#pragma unroll
+      for (int i = 0; i < VN; ++i) {
+        const int vid = tid + 256 * i;
+        if (vid < BN * VPR)
+          *reinterpret_cast<u32x4*>(v_lds + (vid / VPR) * VP +
+                                    (vid % VPR) * VEC) = vreg[i][0];
       }
     }
+  };
+
+  if constexpr (PF) load_tile(0);
+  for (int j0 = 0; j0 <= kv_hi; j0 += BN) {
+    if constexpr (!PF) load_tile(j0);
+    store_tile();
     __syncthreads();
+    if constexpr (PF) {
+      if (j0 + BN <= kv_hi) load_tile(j0 + BN);
+    }
 
     // ---- S^T = K Q^T ----
     const bool interior = wave_full && j0 + BN - 1 <= wave_min_pos;
