@@ -820,9 +820,11 @@ class LatentAttention(nn.Module):
             c.scale, sink=self.sink, value_dims=c.rank, seq_cu=meta.seq_cu,
             tiles=meta.seq_tiles)
         # expand the attended latents: [H, T, rank] x [H, rank, vdim]
-        ov = torch.bmm(o.transpose(0, 1),
-                       self.uv.view(H, c.vdim, c.rank).transpose(1, 2))
-        return self.o_proj(ov.transpose(0, 1).reshape(T, H * c.vdim))
+        ov = torch.empty((T, H, c.vdim), dtype=q.dtype, device=q.device)
+        torch.bmm(o.transpose(0, 1),
+                  self.uv.view(H, c.vdim, c.rank).transpose(1, 2),
+                  out=ov.transpose(0, 1))
+        return self.o_proj(ov.view(T, H * c.vdim))
 
 
 class RGLRUMixer(nn.Module):

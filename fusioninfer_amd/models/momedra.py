@@ -276,21 +276,21 @@ class MomedraLM(nn.Module):
     # ----------------------------------------------------------- forward
     def forward(self, input_ids, meta, caches, hidden=None, residual=None):
         eps = self.arch.eps
-        x0 = self.embed_tokens[input_ids]
-        # a copy also in fp32 mode: the stream is updated in place and the
-        # embedding output is read again at every pass entry
-        resid = x0.to(torch.float32, copy=True)
-        h = None
+        x0 = self.embed_tokens[input_ids].contiguous()
         n = len(self.runs)
+        # the stream starts as an fp32 copy of the embedding output (which
+        # is read again at every pass entry), fused with the first norm
+        # unless the first run enters a pass
+        first = self.layers[self.runs[0][0]]
+        resid, h = seqmix.cast_layer_norm(
+            x0, None if self.runs[0][1] else first.norm1, eps)
         for r, ((i, enters), cache) in enumerate(zip(self.runs, caches)):
             layer = self.layers[i]
             if enters:
                 # x <- W_in [x; embedding output], then this layer's norm
-                xin = torch.cat([resid.to(self.dtype), x0], dim=-1)
-                resid = self.loop_in(xin).float()
-                h = None
-            if h is None:
-                h = seqmix.layer_norm(resid, layer.norm1, eps, self.dtype)
+                xin = seqmix.concat_cast(resid, x0)
+                resid, h = seqmix.cast_layer_norm(self.loop_in(xin),
+                                                  layer.norm1, eps)
             if r + 1 == n:
                 nxt = self.final_norm
             elif self.runs[r + 1][1]:

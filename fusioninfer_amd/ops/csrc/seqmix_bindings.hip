@@ -121,6 +121,11 @@ void launch_rglru_scan(A*, const float*, const float*, const float*,
                        hipStream_t);
 template <typename A>
 void launch_relu_squared(A*, const A*, int64_t, int, int, hipStream_t);
+template <typename A>
+void launch_cast_layer_norm(float*, A*, const A*, const float*, float, int,
+                            int, hipStream_t);
+template <typename A>
+void launch_concat_cast(A*, const float*, const A*, int, int, hipStream_t);
 int sink_attention_splits(int max_keys);
 bool sink_attention_has_tiles(int DK, int DV);
 template <typename A>
@@ -1072,6 +1077,43 @@ void rglru_scan(at::Tensor out, at::Tensor u, at::Tensor gate_lin,
                           stream()));
 }
 
+void cast_layer_norm(at::Tensor resid, c10::optional<at::Tensor> out,
+                     at::Tensor y, c10::optional<at::Tensor> w, double eps) {
+  CHECK_F32(resid);
+  CHECK_ACT(y);
+  TORCH_CHECK(y.dim() == 2 && y.is_contiguous() &&
+              resid.sizes() == y.sizes());
+  TORCH_CHECK(out.has_value() == w.has_value());
+  const float* wp = nullptr;
+  void* op = nullptr;
+  if (w.has_value()) {
+    CHECK_F32(*w);
+    TORCH_CHECK(w->numel() == y.size(1));
+    TORCH_CHECK(out->is_cuda() && out->scalar_type() == y.scalar_type() &&
+                out->sizes() == y.sizes() && out->is_contiguous());
+    wp = w->data_ptr<float>();
+    op = out->data_ptr();
+  }
+  DISPATCH_ACT(y, fi::launch_cast_layer_norm<A>(
+                      resid.data_ptr<float>(), reinterpret_cast<A*>(op),
+                      ptr<A>(y), wp, (float)eps, (int)y.size(0),
+                      (int)y.size(1), stream()));
+}
+
+void concat_cast(at::Tensor out, at::Tensor resid, at::Tensor x0) {
+  CHECK_F32(resid);
+  CHECK_ACT(x0);
+  CHECK_ACT(out);
+  TORCH_CHECK(resid.dim() == 2 && x0.is_contiguous() &&
+              x0.sizes() == resid.sizes() && out.is_contiguous() &&
+              out.scalar_type() == x0.scalar_type() && out.dim() == 2 &&
+              out.size(0) == resid.size(0) &&
+              out.size(1) == 2 * resid.size(1));
+  DISPATCH_ACT(x0, fi::launch_concat_cast<A>(
+                       ptr<A>(out), resid.data_ptr<float>(), ptr<A>(x0),
+                       (int)resid.size(0), (int)resid.size(1), stream()));
+}
+
 void relu_squared(at::Tensor out, at::Tensor x) {
   CHECK_ACT(x);
   CHECK_ACT(out);
@@ -1101,6 +1143,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "per-channel causal convolution with the tail kept per sequence");
   m.def("rglru_scan", &rglru_scan, "gated linear recurrence times gelu branch");
   m.def("relu_squared", &relu_squared, "relu(x)^2");
+  m.def("cast_layer_norm", &cast_layer_norm,
+        "fp32 stream restarted from an activation, then layer norm");
+  m.def("concat_cast", &concat_cast, "[round(stream) | x0] rows");
   m.def("layer_norm", &layer_norm, "layer norm of an fp32 stream, no bias");
   m.def("gated_residual_layer_norm", &gated_residual_layer_norm,
         "fp32 residual += y * sigmoid(gate); optional next layer norm");

@@ -66,6 +66,38 @@ __global__ __launch_bounds__(256) void scaled_residual_layer_norm_kernel(
     Act<A>::st(o + i, (row[i] - mean) * rstd * w_next[i]);
 }
 
+// resid (fp32) = y; out = layer_norm(resid) * w: the stream restarts from
+// an activation (embedding rows, the projection that enters a pass)
+template <typename A>
+__global__ __launch_bounds__(256) void cast_layer_norm_kernel(
+    float* __restrict__ resid, A* __restrict__ out, const A* __restrict__ y,
+    const float* __restrict__ w, float eps, int W) {
+  __shared__ float scratch[8];
+  const int64_t t = blockIdx.x;
+  float* row = resid + t * W;
+  for (int i = threadIdx.x; i < W; i += 256)
+    row[i] = Act<A>::ld(y + t * W + i);
+  if (w == nullptr) return;
+  __syncthreads();
+  float mean, rstd;
+  row_moments_p(row, W, eps, scratch, mean, rstd);
+  A* o = out + t * W;
+  for (int i = threadIdx.x; i < W; i += 256)
+    Act<A>::st(o + i, (row[i] - mean) * rstd * w[i]);
+}
+
+// out[t] = [round(resid[t]) | x0[t]]: input rows of the pass-entry product
+template <typename A>
+__global__ __launch_bounds__(256) void concat_cast_kernel(
+    A* __restrict__ out, const float* __restrict__ resid,
+    const A* __restrict__ x0, int W) {
+  const int64_t t = blockIdx.y;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= W) return;
+  Act<A>::st(out + t * 2 * W + i, resid[t * W + i]);
+  out[t * 2 * W + W + i] = x0[t * W + i];
+}
+
 constexpr int kHeadSlots = 8;   // head sizes up to 512
 
 template <typename A>
@@ -373,6 +405,22 @@ void launch_scaled_residual_layer_norm(float* resid, const A* y1, float s1,
 }
 
 template <typename A>
+void launch_cast_layer_norm(float* resid, A* out, const A* y, const float* w,
+                            float eps, int T, int W, hipStream_t st) {
+  if (T == 0) return;
+  hipLaunchKernelGGL(cast_layer_norm_kernel<A>, dim3(T), dim3(256), 0, st,
+                     resid, out, y, w, eps, W);
+}
+
+template <typename A>
+void launch_concat_cast(A* out, const float* resid, const A* x0, int T, int W,
+                        hipStream_t st) {
+  if (T == 0) return;
+  hipLaunchKernelGGL(concat_cast_kernel<A>, dim3(ceil_div(W, 256), T),
+                     dim3(256), 0, st, out, resid, x0, W);
+}
+
+template <typename A>
 void launch_headnorm_qtemp_cache(A* q_out, const A* q, int64_t q_stride,
                                  const A* k, int64_t k_stride, const A* v,
                                  int64_t v_stride, const int* positions,
@@ -461,6 +509,10 @@ void launch_relu_squared(A* out, const A* x, int64_t x_stride, int T, int N,
 }
 
 #define FI_INST(A)                                                             \
+  template void launch_cast_layer_norm<A>(float*, A*, const A*, const float*,  \
+                                          float, int, int, hipStream_t);       \
+  template void launch_concat_cast<A>(A*, const float*, const A*, int, int,    \
+                                      hipStream_t);                            \
   template void launch_scaled_residual_layer_norm<A>(                          \
       float*, const A*, float, const A*, float, const A*, float, const float*, \
       A*, float, int, int, hipStream_t);                                       \

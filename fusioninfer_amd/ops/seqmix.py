@@ -367,6 +367,28 @@ def scaled_residual_layer_norm_(resid, ys, scales, w_next, eps: float,
                                            out_dtype)
 
 
+def cast_layer_norm(y, w_next, eps: float):
+    """Restart the fp32 stream from the activation rows y: returns (fp32
+    copy of y, layer_norm of it times w_next in y's dtype or None)."""
+    if y.is_cuda:
+        resid = torch.empty(y.shape, dtype=torch.float32, device=y.device)
+        out = torch.empty_like(y) if w_next is not None else None
+        _native().cast_layer_norm(resid, out, y, w_next, eps)
+        return resid, out
+    return ref.cast_layer_norm(y, w_next, eps)
+
+
+def concat_cast(resid, x0):
+    """[resid rounded to x0's dtype | x0]: input rows of a product that
+    reads the stream next to an activation."""
+    if resid.is_cuda:
+        out = torch.empty((resid.shape[0], 2 * resid.shape[1]),
+                          dtype=x0.dtype, device=x0.device)
+        _native().concat_cast(out, resid, x0)
+        return out
+    return ref.concat_cast(resid, x0)
+
+
 def headnorm_qtemp_cache_(q, k, v, positions, q_w, k_w, eps: float,
                           temp_coef: float, temp_every: int, k_cache,
                           v_cache, slot_mapping, num_heads: int,

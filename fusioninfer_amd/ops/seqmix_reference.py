@@ -433,6 +433,20 @@ def scaled_residual_layer_norm_(resid, ys, scales, w_next, eps: float,
     return layer_norm(resid, w_next, eps, out_dtype)
 
 
+def cast_layer_norm(y, w_next, eps: float):
+    """The fp32 stream restarted from an activation: returns (y as fp32
+    copy, layer_norm(y) * w_next in y's dtype, or None without w_next)."""
+    resid = y.to(torch.float32, copy=True)
+    if w_next is None:
+        return resid, None
+    return resid, layer_norm(resid, w_next, eps, y.dtype)
+
+
+def concat_cast(resid, x0):
+    """[resid rounded to x0's dtype | x0] along the last dim."""
+    return torch.cat([resid.to(x0.dtype), x0], dim=-1)
+
+
 def query_temperature(positions, coef: float, every: int):
     """1 + coef * ln(floor((p + 1) / every) + 1) per row, fp32 (1 when
     every <= 0)."""

@@ -283,6 +283,20 @@ def test_scaled_residual_and_layer_norm(device):
     assert torch.allclose(resid.cpu(), x + ys[0], atol=1e-6)
     r = seqmix.relu_squared((x - 1.5).to(device)).cpu()
     assert torch.allclose(r, torch.relu(x - 1.5) ** 2, atol=1e-6)
+    # the stream restarted from an activation, and the rows that enter a
+    # pass of a repeated span
+    stream, h = seqmix.cast_layer_norm(x.to(device), w.to(device), 1e-3)
+    assert stream.dtype == torch.float32 and torch.equal(stream.cpu(), x)
+    assert torch.allclose(h.cpu().double(),
+                          oracle.layer_norm(x.double(), w.double(), 1e-3),
+                          atol=1e-5)
+    stream, h = seqmix.cast_layer_norm(x.to(device), None, 1e-3)
+    assert h is None and torch.equal(stream.cpu(), x)
+    xb = ys[0].to(torch.bfloat16)
+    both = seqmix.concat_cast(x.to(device), xb.to(device)).cpu()
+    assert both.dtype == torch.bfloat16 and both.shape == (T, 2 * W_)
+    assert torch.equal(both[:, :W_], x.to(torch.bfloat16))
+    assert torch.equal(both[:, W_:], xb)
 
 
 @pytest.mark.parametrize("device", DEVICES)
