@@ -48,6 +48,19 @@ model designs assemble them freely:
   mixer or several scaled mixers side by side behind ONE merged input
   projection (which also carries the gate's W).
 
+* ``WindowedSinkAttention``  grouped-query softmax attention with
+  projection biases, ONE RMS norm over the whole query (and key)
+  projection, interleaved partial rotary positions whose frequencies can
+  be blended for context extension, a sliding window that always keeps the
+  first keys, a per-head softmax sink and an elementwise sigmoid gate; a
+  layer may read another layer's paged keys and values instead of
+  projecting its own.
+* ``ClampedGatedMLP``    down(g' sigmoid(1.702 g') (u' + 1)) with the gate
+  clamped from above and the up branch on both sides.
+* ``PostNormLayer``      x <- x + LN(mixer(x)), x <- x + LN(ff(x)): the
+  sublayers read the stream itself and the layer norm (weight and bias)
+  sits on their output.
+
 Activations run in the model dtype (bf16 or fp32); statistics, rotary
 angles, scores, decays, gates of the recurrence and the state are fp32
 inside the ops (fusioninfer_amd/ops/seqmix.py).
@@ -465,11 +478,17 @@ class GatedDeltaMixer(nn.Module):
 
 class RoutedExperts(nn.Module):
     """Mixture of feed-forward experts: down(silu(gate x) * up x)
-    (``act`` "silu_gate") or down(relu(up x)^2) (``act`` "relu_sq").
+    (``act`` "silu_gate"), down(relu(up x)^2) (``act`` "relu_sq") or the
+    clamped gated unit down(g' sigmoid(1.702 g') (u' + 1)), g' = min(gate
+    x, limit), u' = clamp(up x, -limit, limit) (``act`` "clamped_glu").
 
     Router logits are an fp32 product (plus an optional bias); scores are sigmoid(z) or
     softmax(z); the ``top`` largest are chosen, optionally divided by their
-    sum (+1e-20), and multiplied by ``scale``. On the GPU the experts run
+    sum (+1e-20), and multiplied by ``scale``. With ``groups`` = (count,
+    keep) the router is group-limited: sigmoid scores, the choice runs on
+    score + a per-expert correction inside the ``keep`` best of ``count``
+    groups of neighbouring experts, and the weights are the chosen scores
+    as they are. On the GPU the experts run
     as two grouped GEMMs over block-aligned expert segments: the MFMA
     kernel on packed bf16 weights where the sizes fit its tiles, the
     plain grouped kernel otherwise (fp32, odd sizes)."""
@@ -477,14 +496,25 @@ class RoutedExperts(nn.Module):
     def __init__(self, width: int, ff: int, experts: int, top: int, dtype,
                  score: str = "sigmoid", renorm: bool = True,
                  scale: float = 1.0, act: str = "silu_gate",
-                 router_bias: bool = False):
+                 router_bias: bool = False, limit: float = 0.0,
+                 groups: Optional[Tuple[int, int]] = None):
         super().__init__()
         if score not in ("sigmoid", "softmax"):
             raise ValueError(f"unknown router score {score!r}")
-        if act not in ("silu_gate", "relu_sq"):
+        if act not in ("silu_gate", "relu_sq", "clamped_glu"):
             raise ValueError(f"unknown expert activation {act!r}")
         self.act = act
-        self.gated = act == "silu_gate"
+        self.gated = act != "relu_sq"
+        self.limit = float(limit)
+        self.groups = None
+        if groups is not None:
+            count, keep = int(groups[0]), int(groups[1])
+            if (count < 1 or experts % count or not 1 <= keep <= count
+                    or top > keep * (experts // count)):
+                raise ValueError(
+                    f"router groups {groups} do not fit {experts} experts "
+                    f"with top {top}")
+            self.groups = (count, keep)
         if not 1 <= top <= experts:
             raise ValueError("top must be in 1..experts")
         self.width, self.ff, self.experts, self.top = width, ff, experts, top
@@ -495,6 +525,9 @@ class RoutedExperts(nn.Module):
             requires_grad=False)
         self.router_bias = (_f32_param((experts,), 0.0) if router_bias
                             else None)
+        # group-limited routing: added to the scores for the choice only
+        self.correction = (_f32_param((experts,), 0.0)
+                           if self.groups is not None else None)
         # gated: gate rows then up rows; otherwise the up rows alone
         self.gate_up = nn.Parameter(
             torch.empty(experts, (2 if self.gated else 1) * ff, width,
@@ -538,6 +571,9 @@ class RoutedExperts(nn.Module):
         from fusioninfer_amd import ops
 
         logits = F.linear(x.float(), self.router, self.router_bias)
+        if self.groups is not None:
+            return ops.moe_route_grouped(logits, self.correction, self.top,
+                                         self.groups[0], self.groups[1])
         return ops.moe_route(logits, self.top, self.score, self.renorm,
                              self.scale)
 
@@ -553,7 +589,9 @@ class RoutedExperts(nn.Module):
                 if rows.numel() == 0:
                     continue
                 gu = F.linear(x[rows], self.gate_up[e]).float()
-                if self.gated:
+                if self.act == "clamped_glu":
+                    act = seqmix.clamped_glu(gu, self.limit).to(x.dtype)
+                elif self.gated:
                     act = (F.silu(gu[:, : self.ff])
                            * gu[:, self.ff:]).to(x.dtype)
                 else:
@@ -570,17 +608,18 @@ class RoutedExperts(nn.Module):
             topi, 0, E, block_m)
         act = torch.empty(PM, self.ff, dtype=x.dtype, device=x.device)
         y = torch.empty(PM, self.width, dtype=x.dtype, device=x.device)
+        up_act = None if self.act == "silu_gate" else self.act
         if fast:
             gu_p, dn_p = self._packed_weights()
             ops.moe_gemm(act, x, gu_p, sorted_ids, expert_ids, n_valid,
-                         block_m, gate_up=self.gated,
-                         up_act=None if self.gated else "relu_sq")
+                         block_m, gate_up=self.gated, up_act=up_act,
+                         limit=self.limit)
             ops.moe_gemm(y, act, dn_p, sorted_ids, expert_ids, n_valid,
                          block_m, gate_up=False)
         else:
             ops.moe_gemm_plain(act, x, self.gate_up, sorted_ids, expert_ids,
                                n_valid, block_m, gate_up=self.gated,
-                               up_act=None if self.gated else "relu_sq")
+                               up_act=up_act, limit=self.limit)
             ops.moe_gemm_plain(y, act, self.down, sorted_ids, expert_ids,
                                n_valid, block_m, gate_up=False)
         out = torch.empty(T, self.width, dtype=x.dtype, device=x.device)
@@ -949,3 +988,166 @@ class ParallelResidualLayer(nn.Module):
         return seqmix.scaled_residual_layer_norm_(
             resid, ys, [self.mult] * len(ys), next_norm_w, self.eps,
             self.dtype)
+
+
+# ------------------------------------------------------------------------
+# Post-norm family of blocks
+
+
+@dataclasses.dataclass
+class WindowedSinkAttentionConfig:
+    heads: int
+    kv_heads: int
+    dim: int                 # per-head query/key size
+    vdim: int                # per-head value size
+    scale: float             # score multiplier
+    window: int = 0          # 0: plain causal; else p - j < window ...
+    keep_first: int = 0      # ... or j < keep_first
+    rot_dims: int = 0        # leading entries of a head that turn (0: none)
+    rot_base: float = 10000.0
+    # frequency blend for context extension (rot_original 0: none)
+    rot_factor: float = 1.0
+    rot_original: float = 0.0
+    rot_fast: float = 0.0
+    rot_slow: float = 0.0
+
+    def __post_init__(self):
+        if self.heads % self.kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        if self.rot_dims % 2 or self.rot_dims > self.dim:
+            raise ValueError("rot.dims must be even and at most dim")
+        if self.window < 0 or self.keep_first < 0:
+            raise ValueError("window and keep_first must not be negative")
+
+
+class WindowedSinkAttention(nn.Module):
+    """q, k, v and the elementwise gate come from the caller's merged
+    projection (the gate's rows carry a zero bias). With ``own_kv`` False
+    the block has neither key nor value branches and ``forward`` is handed
+    the cache of the layer it borrows from."""
+
+    has_bias = True
+    biased = ("q", "k", "v")
+
+    def __init__(self, cfg: WindowedSinkAttentionConfig, width: int,
+                 eps: float, dtype, own_kv: bool = True):
+        super().__init__()
+        self.cfg = cfg
+        self.eps = eps
+        self.dtype = dtype
+        self.own_kv = own_kv
+        H, G = cfg.heads, cfg.kv_heads
+        if own_kv:
+            self.in_names = ["q", "k", "v", "g"]
+            self.in_sizes = [H * cfg.dim, G * cfg.dim, G * cfg.vdim,
+                             H * cfg.vdim]
+        else:
+            self.in_names = ["q", "g"]
+            self.in_sizes = [H * cfg.dim, H * cfg.vdim]
+        self.q_norm = _f32_param((H * cfg.dim,), 1.0)
+        self.k_norm = _f32_param((G * cfg.dim,), 1.0) if own_kv else None
+        self.sink = _f32_param((H,), 0.0)
+        self.o_proj = RowParallelLinear(H * cfg.vdim, width, dtype=dtype)
+        if cfg.rot_dims:
+            inv_freq, mult = seqmix.blended_rotary(
+                cfg.rot_dims, cfg.rot_base, cfg.rot_factor, cfg.rot_original,
+                cfg.rot_fast, cfg.rot_slow)
+        else:
+            inv_freq, mult = torch.zeros(0, dtype=torch.float32), 1.0
+        self.rot_mult = float(mult)
+        self.register_buffer("inv_freq", inv_freq, persistent=False)
+
+    def state_tensors(self, num_blocks, block_size, num_slots, device):
+        if not self.own_kv:
+            return {}
+        c = self.cfg
+        return {
+            "k": torch.zeros((num_blocks, c.kv_heads, block_size, c.dim),
+                             dtype=self.dtype, device=device),
+            "v": torch.zeros((num_blocks, c.kv_heads, block_size, c.vdim),
+                             dtype=self.dtype, device=device),
+        }
+
+    def block_bytes(self, block_size: int) -> int:
+        if not self.own_kv:
+            return 0
+        c = self.cfg
+        esize = torch.empty((), dtype=self.dtype).element_size()
+        return c.kv_heads * block_size * (c.dim + c.vdim) * esize
+
+    def forward(self, parts, meta, cache) -> torch.Tensor:
+        c = self.cfg
+        if self.own_kv:
+            q, k, v, g = parts
+        else:
+            (q, g), k, v = parts, None, None
+        qn = seqmix.widenorm_rope_cache_(
+            q, k, v, meta.positions, self.q_norm, self.k_norm, self.eps,
+            self.inv_freq, self.rot_mult, cache["k"], cache["v"],
+            meta.slot_mapping, c.heads, c.kv_heads, c.dim, c.vdim)
+        o = seqmix.sink_paged_attention(
+            qn, cache["k"], cache["v"], meta.seq_bt, meta.row_seq,
+            meta.positions, c.scale, sink=self.sink, out_gate=g,
+            seq_cu=meta.seq_cu, tiles=meta.seq_tiles, window=c.window,
+            keep_first=c.keep_first)
+        return self.o_proj(o.view(o.shape[0], c.heads * c.vdim))
+
+
+class ClampedGatedMLP(nn.Module):
+    """down(g' sigmoid(1.702 g') (u' + 1)), g' = min(gate x, limit),
+    u' = clamp(up x, -limit, limit); gate and up are one merged GEMM."""
+
+    def __init__(self, width: int, ff: int, limit: float, dtype):
+        super().__init__()
+        self.ff = ff
+        self.limit = float(limit)
+        self.gate_up_proj = MergedColumnParallelLinear(width, [ff, ff],
+                                                       dtype=dtype)
+        self.down_proj = RowParallelLinear(ff, width, dtype=dtype)
+
+    def forward(self, x):
+        return self.down_proj(
+            seqmix.clamped_glu(self.gate_up_proj(x), self.limit))
+
+
+class PostNormLayer(nn.Module):
+    """x <- x + LN1(mixer(x)); x <- x + LN2(ff(x)) on an fp32 stream x.
+    The sublayers read x itself (rounded to the activation dtype); the
+    layer norms carry weight and bias and sit on the sublayer outputs, so
+    each is one kernel with the residual sum. ``forward`` receives and
+    returns the activation-dtype copy of the stream."""
+
+    def __init__(self, mixer: nn.Module, mlp: Optional[nn.Module],
+                 width: int, eps: float, dtype):
+        super().__init__()
+        self.mixer = mixer
+        self.mlp = mlp
+        self.eps = eps
+        self.dtype = dtype
+        self.branches: List[str] = list(mixer.in_names)
+        self.sizes: List[int] = list(mixer.in_sizes)
+        self.in_proj = MergedColumnParallelLinear(
+            width, self.sizes, dtype=dtype, bias=mixer.has_bias)
+        self.norm1 = _f32_param((width,), 1.0)
+        self.norm1_b = _f32_param((width,), 0.0)
+        if mlp is not None:
+            self.norm2 = _f32_param((width,), 1.0)
+            self.norm2_b = _f32_param((width,), 0.0)
+
+    def in_proj_rows(self, branch: str):
+        off = 0
+        for name, size in zip(self.branches, self.sizes):
+            if name == branch:
+                return off, size
+            off += size
+        raise KeyError(branch)
+
+    def forward(self, resid, x, meta, cache):
+        parts = self.in_proj(x).split(self.sizes, dim=-1)
+        y = self.mixer(parts, meta, cache)
+        x = seqmix.post_norm_residual_(resid, y, self.norm1, self.norm1_b,
+                                       self.eps, self.dtype)
+        if self.mlp is None:
+            return x
+        return seqmix.post_norm_residual_(resid, self.mlp(x), self.norm2,
+                                          self.norm2_b, self.eps, self.dtype)

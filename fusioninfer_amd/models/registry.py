@@ -267,6 +267,19 @@ def _register_builtin_architectures() -> None:
     register_architecture("Momedra", momedra_config, momedra_model,
                           extensions=("seqmix", "moe"))
 
+    def kazozen_config(raw, model_path):
+        from fusioninfer_amd.models import kazozen
+
+        return kazozen.model_config_from_dict(raw, model_path)
+
+    def kazozen_model(cfg):
+        from fusioninfer_amd.models.kazozen import KazozenLM
+
+        return KazozenLM(cfg)
+
+    register_architecture("Kazozen", kazozen_config, kazozen_model,
+                          extensions=("seqmix", "moe"))
+
 
 _register_builtin_architectures()
 

@@ -388,16 +388,21 @@ def has_moe_native() -> bool:
 
 def _moe_gemm_mode(gate_up: bool, up_act) -> int:
     """0: plain GEMM over act rows; 1: gathered x rows, gate|up columns,
-    silu(gate) * up; 2: gathered x rows, up columns alone, relu(up)^2."""
+    silu(gate) * up; 2: gathered x rows, up columns alone, relu(up)^2;
+    3: gathered x rows, gate|up columns, clamped gated unit
+    g' sigmoid(1.702 g') (u' + 1) with g' = min(g, limit),
+    u' = clamp(u, -limit, limit)."""
     if up_act is None:
         return 1 if gate_up else 0
+    if up_act == "clamped_glu" and gate_up:
+        return 3
     if up_act != "relu_sq" or gate_up:
         raise ValueError(f"unsupported expert activation {up_act!r}")
     return 2
 
 
 def moe_gemm(out, a, b_packed, sorted_ids, expert_ids, n_valid,
-             block_m: int, gate_up: bool, up_act=None):
+             block_m: int, gate_up: bool, up_act=None, limit: float = 0.0):
     """Grouped GEMM over block-aligned expert segments.
 
     out [PM, N] bf16; a = x [T, K] (gate_up, rows gathered via sorted_ids)
@@ -406,25 +411,28 @@ def moe_gemm(out, a, b_packed, sorted_ids, expert_ids, n_valid,
     the real m-tile count (static grid, dynamic work — hipGraph-safe).
     gate_up=True fuses the SwiGLU epilogue: out = silu(gate) * up.
     up_act="relu_sq" (with gate_up=False): a = x gathered like gate_up,
-    b holds the up matrix alone and out = relu(a @ up)^2."""
+    b holds the up matrix alone and out = relu(a @ up)^2.
+    up_act="clamped_glu" (with gate_up=True): the gated unit clamps gate
+    from above and up on both sides at ``limit`` (see _moe_gemm_mode)."""
     mode = _moe_gemm_mode(gate_up, up_act)
     if out.is_cuda:
         _moe_native().moe_gemm(out, a, b_packed, sorted_ids, expert_ids,
-                               n_valid, block_m, mode)
+                               n_valid, block_m, mode, float(limit))
         return out
     return ref.moe_gemm(out, a, b_packed, sorted_ids, expert_ids, n_valid,
-                        block_m, gate_up, up_act)
+                        block_m, gate_up, up_act, limit)
 
 
 def moe_gemm_plain(out, a, w, sorted_ids, expert_ids, n_valid, block_m: int,
-                   gate_up: bool, up_act=None):
+                   gate_up: bool, up_act=None, limit: float = 0.0):
     """Grouped GEMM of the same block-aligned layout for ANY sizes and for
     fp32 or bf16 operands (fp32 accumulation): w is the experts' natural
     [E, out, in] weight ([E, 2N, K] with gate rows first when gate_up,
     which also applies out = silu(gate) * up; up_act="relu_sq": [E, N, K]
     up rows alone on gathered x rows, out = relu(.)^2). GPU only."""
     _moe_native().moe_gemm_plain(out, a, w, sorted_ids, expert_ids, n_valid,
-                                 block_m, _moe_gemm_mode(gate_up, up_act))
+                                 block_m, _moe_gemm_mode(gate_up, up_act),
+                                 float(limit))
     return out
 
 
@@ -496,6 +504,29 @@ def moe_route(logits: torch.Tensor, k: int, score: str = "softmax",
                                 score == "sigmoid", renorm, float(scale))
         return topv, topi
     return ref.moe_route(logits, k, score, renorm, scale)
+
+
+def moe_route_grouped(logits: torch.Tensor, correction: torch.Tensor,
+                      k: int, groups: int = 1, keep: int = 1):
+    """Group-limited router tail: s = sigmoid(logits) in fp32; the choice
+    runs on s + correction, restricted to the experts of the ``keep`` best
+    of ``groups`` equal groups of neighbouring experts (group score = sum
+    of its two largest choice scores); weights = the chosen s, not
+    renormalised. Returns (weights [T,k] fp32, ids [T,k] int32)."""
+    E = logits.shape[1]
+    if groups < 1 or E % groups or not 1 <= keep <= groups:
+        raise ValueError("experts must split into equal groups, "
+                         "1 <= keep <= groups")
+    if k > keep * (E // groups):
+        raise ValueError("top exceeds the experts of the kept groups")
+    if logits.is_cuda:
+        T = logits.shape[0]
+        topv = torch.empty(T, k, dtype=torch.float32, device=logits.device)
+        topi = torch.empty(T, k, dtype=torch.int32, device=logits.device)
+        _moe_native().moe_route_grouped(logits.contiguous(), correction,
+                                        topv, topi, k, groups, keep)
+        return topv, topi
+    return ref.moe_route_grouped(logits, correction, k, groups, keep)
 
 
 def moe_combine(out, y, pos, w):

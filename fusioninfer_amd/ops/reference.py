@@ -313,7 +313,7 @@ def unpack_moe_weights(b_packed: torch.Tensor) -> torch.Tensor:
 
 
 def moe_gemm(out, a, b_packed, sorted_ids, expert_ids, n_valid,
-             block_m: int, gate_up: bool, up_act=None):
+             block_m: int, gate_up: bool, up_act=None, limit: float = 0.0):
     """fp32 reference of the grouped GEMM (CPU; same semantics as the HIP
     kernel incl. padding rows computed from the dummy token row)."""
     w = unpack_moe_weights(b_packed).float()
@@ -328,7 +328,11 @@ def moe_gemm(out, a, b_packed, sorted_ids, expert_ids, n_valid,
         else:
             src = a[rows].float()
         acc = src @ w[e]
-        if gate_up:
+        if gate_up and up_act == "clamped_glu":
+            g = acc[:, :N].clamp(max=limit)
+            u = acc[:, N:].clamp(-limit, limit)
+            acc = g * torch.sigmoid(1.702 * g) * (u + 1.0)
+        elif gate_up:
             g, u = acc[:, :N], acc[:, N:]
             acc = torch.nn.functional.silu(g) * u
         elif up_act == "relu_sq":
@@ -377,6 +381,27 @@ def moe_gemm_fp8(out, a, a_scales, b_packed, b_scales, sorted_ids,
             acc = torch.nn.functional.silu(g) * u
         out[rows] = acc.to(out.dtype)
     return out
+
+
+def moe_route_grouped(logits, correction, k: int, groups: int, keep: int):
+    """Group-limited router tail: scores s = sigmoid(logits); the choice
+    runs on s + correction, the weights are the chosen s (no
+    renormalisation). Experts form ``groups`` equal groups of neighbours; a
+    group's score is the sum of its two largest choice scores and only
+    experts of the ``keep`` best groups can be chosen."""
+    z = logits.float()
+    s = torch.sigmoid(z)
+    c = s + correction.float()
+    T, E = z.shape
+    if groups > 1 and keep < groups:
+        n = E // groups
+        cg = c.view(T, groups, n)
+        gs = cg.topk(min(2, n), dim=-1).values.sum(-1)
+        kept = torch.zeros(T, groups, dtype=torch.bool)
+        kept.scatter_(1, gs.topk(keep, dim=-1).indices, True)
+        c = cg.masked_fill(~kept[:, :, None], float("-inf")).reshape(T, E)
+    topi = c.topk(k, dim=-1).indices
+    return s.gather(1, topi), topi.int()
 
 
 def moe_route(logits, k: int, score: str, renorm: bool, scale: float):

@@ -431,12 +431,15 @@ SPLIT_ROWS_PER_LAUNCH = 512  # rows per launch of the split attention form
 
 def sink_paged_attention(q, k_cache, v_cache, seq_bt, row_seq, positions,
                          scale: float, sink=None, value_dims: int = 0,
-                         out_gate=None, seq_cu=None, tiles=None):
+                         out_gate=None, seq_cu=None, tiles=None,
+                         window: int = 0, keep_first: int = 0):
     """Causal softmax attention over the paged cache with separate key and
     value sizes, an optional per-head sink in the denominator, values that
     may be the leading ``value_dims`` entries of the cached keys
-    (``v_cache`` None) and an optional sigmoid gate per (row, head) on the
-    result. ``tiles`` as for ranged_paged_attention."""
+    (``v_cache`` None) and an optional sigmoid gate on the result, per
+    (row, head) ([T, H]) or per entry ([T, H*Dv]). ``window`` > 0 hides
+    key j from position p unless p - j < window or j < keep_first.
+    ``tiles`` as for ranged_paged_attention."""
     if q.is_cuda:
         T, H, _ = q.shape
         V = v_cache.shape[3] if v_cache is not None else int(value_dims)
@@ -462,11 +465,11 @@ def sink_paged_attention(q, k_cache, v_cache, seq_bt, row_seq, positions,
                                        row_seq, positions, float(scale),
                                        sink, V, out_gate, seq_cu, tile_seq,
                                        tile_row0, int(tile_rows), part_ml,
-                                       part_o)
+                                       part_o, int(window), int(keep_first))
         return out
     return ref.sink_paged_attention(q, k_cache, v_cache, seq_bt, row_seq,
                                     positions, scale, sink, value_dims,
-                                    out_gate)
+                                    out_gate, window, keep_first)
 
 
 def causal_conv_state(x, conv_w, conv_b, conv_state, seq_cu, row_seq,
@@ -504,3 +507,96 @@ def relu_squared(x):
         _native().relu_squared(out, x)
         return out
     return ref.relu_squared(x)
+
+
+# ------------------------------------------------------------------------
+# post-norm stream with a token-pair embedding, whole-projection q/k norm
+# with blended rotary frequencies, clamped gated unit, capped logits
+
+blended_rotary = ref.blended_rotary
+
+
+def pair_embed(ids, embed, embed_scale: float, pair_table, buckets: int,
+               mul_prev: int, mul_cur: int, prev_token, seq_cu, seq_slots,
+               positions, act_dtype):
+    """Start of an fp32 stream: embed[id] * embed_scale plus the pair
+    table's row for (previous id, id) (row ``buckets`` at position 0). The
+    previous id of a group's first row is read from ``prev_token`` [slots]
+    int32, which then receives the group's last id. Returns (fp32 stream,
+    its rounding to act_dtype)."""
+    if embed.is_cuda:
+        T, W = ids.shape[0], embed.shape[1]
+        resid = torch.empty((T, W), dtype=torch.float32, device=embed.device)
+        act = (resid if act_dtype == torch.float32 else
+               torch.empty((T, W), dtype=act_dtype, device=embed.device))
+        _native().pair_embed(resid, act, ids, embed, float(embed_scale),
+                             pair_table, int(buckets), int(mul_prev),
+                             int(mul_cur), prev_token, seq_cu, seq_slots,
+                             positions)
+        return resid, act
+    return ref.pair_embed(ids, embed, embed_scale, pair_table, buckets,
+                          mul_prev, mul_cur, prev_token, seq_cu, seq_slots,
+                          positions, act_dtype)
+
+
+def layer_norm_affine(x, w, b, eps: float, out_dtype):
+    """(x - mean) / sqrt(var + eps) * w + b with fp32 statistics."""
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        _native().layer_norm_affine(out, x, w, b, eps)
+        return out
+    return ref.layer_norm_affine(x, w, b, eps, out_dtype)
+
+
+def post_norm_residual_(resid, y, w, b, eps: float, out_dtype):
+    """resid (fp32, in place) += layer_norm(y) * w + b, the norm sitting on
+    the sublayer's OUTPUT y; returns resid rounded to out_dtype (resid
+    itself for fp32), the next sublayer's input."""
+    if resid.is_cuda:
+        out = (resid if out_dtype == torch.float32 else
+               torch.empty(resid.shape, dtype=out_dtype, device=resid.device))
+        _native().post_norm_residual(resid, y, w, b, out, eps)
+        return out
+    return ref.post_norm_residual_(resid, y, w, b, eps, out_dtype)
+
+
+def widenorm_rope_cache_(q, k, v, positions, q_w, k_w, eps: float, inv_freq,
+                         rot_mult: float, k_cache, v_cache, slot_mapping,
+                         num_heads: int, num_kv_heads: int, dim: int,
+                         vdim: int):
+    """RMS norm over the whole q (and k) row times a weight vector, then
+    interleaved-pair rotation of the leading 2*len(inv_freq) entries of
+    every head (cos/sin times rot_mult); processed k and raw v go into the
+    paged caches. ``k`` None: queries only. q/k/v may be column slices of
+    one projection output; returns a fresh contiguous q [T, H, dim]."""
+    if q.is_cuda:
+        out = torch.empty((q.shape[0], num_heads, dim), dtype=q.dtype,
+                          device=q.device)
+        _native().widenorm_rope_cache(out, q, k, v, positions, q_w, k_w, eps,
+                                      inv_freq, float(rot_mult), k_cache,
+                                      v_cache, slot_mapping, num_heads,
+                                      num_kv_heads, dim, vdim)
+        return out
+    return ref.widenorm_rope_cache_(q, k, v, positions, q_w, k_w, eps,
+                                    inv_freq, rot_mult, k_cache, v_cache,
+                                    slot_mapping, num_heads, num_kv_heads,
+                                    dim, vdim)
+
+
+def clamped_glu(gu, limit: float):
+    """[T, 2F] (gate | up) -> [T, F]: g' sigmoid(1.702 g') (u' + 1) with
+    g' = min(g, limit), u' = clamp(u, -limit, limit)."""
+    if gu.is_cuda:
+        out = torch.empty((gu.shape[0], gu.shape[1] // 2), dtype=gu.dtype,
+                          device=gu.device)
+        _native().clamped_glu(out, gu, float(limit))
+        return out
+    return ref.clamped_glu(gu, limit)
+
+
+def tanh_cap_(logits, cap: float):
+    """fp32 logits, in place: cap * tanh(logits / cap)."""
+    if logits.is_cuda:
+        _native().tanh_cap(logits, float(cap))
+        return logits
+    return ref.tanh_cap_(logits, cap)

@@ -513,13 +513,15 @@ def latent_rope_cache_(q, ckr, positions, inv_freq, norm_w, eps: float,
 
 def sink_paged_attention(q, k_cache, v_cache, seq_bt, row_seq, positions,
                          scale: float, sink=None, value_dims: int = 0,
-                         out_gate=None):
+                         out_gate=None, window: int = 0, keep_first: int = 0):
     """Causal softmax attention of every row over the paged keys 0..p of
     its own sequence. ``sink`` [H] fp32: exp(sink_h) joins the softmax
     denominator (no key, no value). ``v_cache`` None: the values are the
-    leading ``value_dims`` entries of the cached keys. ``out_gate`` [T, H]:
-    head results are multiplied by sigmoid(out_gate). q [T, H, Dk];
-    returns [T, H, Dv]."""
+    leading ``value_dims`` entries of the cached keys. ``out_gate`` [T, H]
+    or [T, H*Dv]: head results (or every entry) are multiplied by
+    sigmoid(out_gate). ``window`` > 0: key j is visible from position p
+    only if p - j < window or j < keep_first. q [T, H, Dk]; returns
+    [T, H, Dv]."""
     T, H, D = q.shape
     G, bs = k_cache.shape[1], k_cache.shape[2]
     rep = H // G
@@ -544,6 +546,9 @@ def sink_paged_attention(q, k_cache, v_cache, seq_bt, row_seq, positions,
         pr = torch.tensor(pos[t:e + 1])
         sc = torch.einsum("ihd,jhd->hij", qf[t:e + 1], kk) * scale
         vis = idx[None, :] <= pr[:, None]
+        if window > 0:
+            vis &= ((pr[:, None] - idx[None, :] < window)
+                    | (idx[None, :] < keep_first))
         sc = sc.masked_fill(~vis[None], float("-inf"))
         m = sc.max(dim=-1, keepdim=True).values
         if sink is not None:
@@ -555,7 +560,9 @@ def sink_paged_attention(q, k_cache, v_cache, seq_bt, row_seq, positions,
         out[t:e + 1] = torch.einsum("hij,jhd->ihd", ex / den, vv)
         t = e + 1
     if out_gate is not None:
-        out = out * torch.sigmoid(out_gate.float()).reshape(T, H, 1)
+        per_head = out_gate.shape[-1] == H
+        out = out * torch.sigmoid(out_gate.float()).reshape(
+            T, H, 1 if per_head else V)
     return out.to(q.dtype)
 
 
@@ -632,3 +639,133 @@ def gelu_tanh(x):
 def relu_squared(x):
     xf = torch.relu(x.float())
     return (xf * xf).to(x.dtype)
+
+
+# ------------------------------------------------------------------------
+# post-norm stream with a token-pair embedding, whole-projection q/k norm
+# with blended rotary frequencies, windowed attention that keeps the first
+# keys, clamped gated unit, capped logits
+
+def pair_embed(ids, embed, embed_scale: float, pair_table, buckets: int,
+               mul_prev: int, mul_cur: int, prev_token, seq_cu, seq_slots,
+               positions, act_dtype):
+    """x = embed[id] * embed_scale + pair_table[(prev * mul_prev + id *
+    mul_cur) mod buckets]; a sequence's first token takes row ``buckets``.
+    The previous token of a group's first row comes from ``prev_token``
+    [slots] int32, which then receives the group's last id. Returns (fp32
+    stream, its rounding to act_dtype). ``pair_table`` None: no pair term."""
+    x = embed[ids.long()].float() * embed_scale
+    cu = seq_cu.tolist()
+    idl = ids.long()
+    if pair_table is not None:
+        prev = torch.empty_like(idl)
+        prev[1:] = idl[:-1]
+        first = torch.zeros_like(idl, dtype=torch.bool)
+        for s in range(len(cu) - 1):
+            a, b = cu[s], cu[s + 1]
+            if b <= a:
+                continue
+            slot = int(seq_slots[s])
+            prev[a] = int(prev_token[slot]) if slot >= 0 else 0
+            first[a] = True
+        row = (prev * mul_prev + idl * mul_cur) % buckets
+        row = torch.where(positions.long() == 0,
+                          torch.full_like(row, buckets), row)
+        x = x + pair_table[row].float()
+    for s in range(len(cu) - 1):
+        a, b = cu[s], cu[s + 1]
+        if b > a and int(seq_slots[s]) >= 0:
+            prev_token[int(seq_slots[s])] = int(ids[b - 1])
+    return x, x.to(act_dtype)
+
+
+def layer_norm_affine(x, w, b, eps: float, out_dtype):
+    xf = x.float()
+    mu = xf.mean(-1, keepdim=True)
+    var = (xf - mu).pow(2).mean(-1, keepdim=True)
+    return ((xf - mu) * torch.rsqrt(var + eps) * w.float()
+            + b.float()).to(out_dtype)
+
+
+def post_norm_residual_(resid, y, w, b, eps: float, out_dtype):
+    """resid (fp32, in place) += layer_norm(y) * w + b; returns resid
+    rounded to out_dtype (the next sublayer's input)."""
+    resid += layer_norm_affine(y, w, b, eps, torch.float32)
+    return resid.to(out_dtype)
+
+
+def blended_rotary(dims: int, base: float, factor: float = 1.0,
+                   original: float = 0.0, fast: float = 0.0,
+                   slow: float = 0.0):
+    """([dims/2] fp32 angular frequencies, factor on cos and sin). With
+    ``factor`` != 1 every frequency f_i is blended between f_i (pairs that
+    turn more than ``fast`` times over ``original`` positions) and
+    f_i / factor (fewer than ``slow`` turns), linearly in the pair index
+    in between, and cos/sin grow by 0.1 ln(factor) + 1."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64),
+                  -2.0 * i / dims)
+    if not original:
+        return f.float(), 1.0
+
+    def index_of(turns):
+        return (dims * math.log(original / (2.0 * math.pi * turns))
+                / (2.0 * math.log(base)))
+
+    lo = max(math.floor(index_of(fast)), 0)
+    hi = min(math.ceil(index_of(slow)), dims - 1)
+    ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    f = f / factor * ramp + f * (1.0 - ramp)
+    return f.float(), 0.1 * math.log(factor) + 1.0
+
+
+def widenorm_rope_cache_(q, k, v, positions, q_w, k_w, eps: float, inv_freq,
+                         rot_mult: float, k_cache, v_cache, slot_mapping,
+                         num_heads: int, num_kv_heads: int, dim: int,
+                         vdim: int):
+    """RMS norm over the WHOLE q row (all heads at once) times q_w, then
+    interleaved-pair rotation of the first 2*len(inv_freq) entries of every
+    head by p * inv_freq with cos/sin times rot_mult; the same for k, which
+    goes into the paged k cache next to the raw v. ``k`` None: only the
+    queries (a layer that reads another layer's cache). Returns q
+    [T, H, dim]."""
+    T = q.shape[0]
+    ang = positions.float()[:, None] * inv_freq.float()[None, :]
+    cos = (torch.cos(ang) * rot_mult)[:, None, :]
+    sin = (torch.sin(ang) * rot_mult)[:, None, :]
+    nrot = 2 * inv_freq.numel()
+
+    def turn(x, w, heads):
+        x = (_rms(x.float(), eps) * w.float()).view(T, heads, dim)
+        a, b = x[..., 0:nrot:2], x[..., 1:nrot:2]
+        out = x.clone()
+        out[..., 0:nrot:2] = a * cos - b * sin
+        out[..., 1:nrot:2] = b * cos + a * sin
+        return out
+
+    qn = turn(q, q_w, num_heads).to(q.dtype)
+    if k is not None:
+        kn = turn(k, k_w, num_kv_heads)
+        bs = k_cache.shape[2]
+        slots = slot_mapping.long()
+        ok = slots >= 0
+        k_cache[slots[ok] // bs, :, slots[ok] % bs, :] = kn[ok].to(
+            k_cache.dtype)
+        v_cache[slots[ok] // bs, :, slots[ok] % bs, :] = v.reshape(
+            T, num_kv_heads, vdim)[ok].to(v_cache.dtype)
+    return qn
+
+
+def clamped_glu(gu, limit: float):
+    """[T, 2F] (gate | up) -> g' sigmoid(1.702 g') (u' + 1) with
+    g' = min(g, limit), u' = clamp(u, -limit, limit)."""
+    ff = gu.shape[1] // 2
+    g = gu[:, :ff].float().clamp(max=limit)
+    u = gu[:, ff:].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)).to(gu.dtype)
+
+
+def tanh_cap_(logits, cap: float):
+    """logits (fp32, in place) <- cap * tanh(logits / cap)."""
+    logits.copy_(cap * torch.tanh(logits / cap))
+    return logits
