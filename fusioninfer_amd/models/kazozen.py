@@ -268,7 +268,7 @@ class KazozenLM(nn.Module):
             input_ids, self.embed_tokens, a.embed_scale, self.pair_table,
             p.buckets if p else 1, p.mul_prev if p else 0,
             p.mul_cur if p else 0, caches[0]["prev_token"], meta.seq_cu,
-            meta.seq_slots, meta.positions, self.dtype)
+            meta.row_seq, meta.seq_slots, meta.positions, self.dtype)
         for layer, cache in zip(self.layers, caches):
             x = layer(resid, x, meta, cache)
             if self.residual_trace is not None:

@@ -51,6 +51,7 @@ SEQMIX_SOURCES = [
     "seqmix_window.hip",
     "seqmix_parallel.hip",
     "seqmix_sink.hip",
+    "seqmix_postnorm.hip",
 ]
 
 EXTENSIONS = {

@@ -13,7 +13,9 @@
 namespace fi {
 
 void launch_moe_gemm(u16*, const u16*, const u16*, const int*, const int*,
-                     const int*, int, int, int, int, int, hipStream_t);
+                     const int*, int, int, int, int, int, float, hipStream_t);
+void launch_moe_route_grouped(const float*, const float*, float*, int*, int,
+                              int, int, int, int, hipStream_t);
 void launch_moe_gemm_fp8(u16*, const unsigned char*, const float*,
                          const unsigned char*, const float*, const int*,
                          const int*, const int*, int, int, int, int, bool,
@@ -29,7 +31,8 @@ void launch_moe_combine(A*, const A*, const int*, const float*, int, int,
                         int, hipStream_t);
 template <typename A>
 void launch_moe_gemm_plain(A*, const A*, const A*, const int*, const int*,
-                           const int*, int, int, int, int, int, hipStream_t);
+                           const int*, int, int, int, int, int, float,
+                           hipStream_t);
 
 }  // namespace fi
 
@@ -52,11 +55,12 @@ hipStream_t current_stream() {
 
 void moe_gemm(at::Tensor out, at::Tensor a, at::Tensor b_packed,
               at::Tensor sorted_ids, at::Tensor expert_ids,
-              at::Tensor n_valid, int64_t block_m, int64_t mode) {
+              at::Tensor n_valid, int64_t block_m, int64_t mode,
+              double limit) {
   // mode 0: plain; 1: gathered rows, silu(gate) * up; 2: gathered rows,
-  // relu(up)^2
-  TORCH_CHECK(mode >= 0 && mode <= 2, "unknown grouped GEMM mode");
-  const bool gate_up = mode == 1;
+  // relu(up)^2; 3: gathered rows, clamped gated unit with `limit`
+  TORCH_CHECK(mode >= 0 && mode <= 3, "unknown grouped GEMM mode");
+  const bool gate_up = mode == 1 || mode == 3;
   CHECK_BF16_CUDA(out);
   CHECK_BF16_CUDA(a);
   CHECK_BF16_CUDA(b_packed);
@@ -86,7 +90,7 @@ void moe_gemm(at::Tensor out, at::Tensor a, at::Tensor b_packed,
                       bf16_cptr(b_packed), sorted_ids.data_ptr<int>(),
                       expert_ids.data_ptr<int>(), n_valid.data_ptr<int>(),
                       PM / block_m, K, N, static_cast<int>(block_m),
-                      static_cast<int>(mode),
+                      static_cast<int>(mode), static_cast<float>(limit),
                       current_stream());
 }
 
@@ -151,9 +155,10 @@ void moe_combine(at::Tensor out, at::Tensor y, at::Tensor pos, at::Tensor w) {
 
 void moe_gemm_plain(at::Tensor out, at::Tensor a, at::Tensor w,
                     at::Tensor sorted_ids, at::Tensor expert_ids,
-                    at::Tensor n_valid, int64_t block_m, int64_t mode) {
-  TORCH_CHECK(mode >= 0 && mode <= 2, "unknown grouped GEMM mode");
-  const bool gate_up = mode == 1;
+                    at::Tensor n_valid, int64_t block_m, int64_t mode,
+                    double limit) {
+  TORCH_CHECK(mode >= 0 && mode <= 3, "unknown grouped GEMM mode");
+  const bool gate_up = mode == 1 || mode == 3;
   TORCH_CHECK(out.is_cuda() && a.is_cuda() && w.is_cuda());
   TORCH_CHECK(out.scalar_type() == a.scalar_type() &&
               out.scalar_type() == w.scalar_type() &&
@@ -177,13 +182,39 @@ void moe_gemm_plain(at::Tensor out, at::Tensor a, at::Tensor w,
     fi::launch_moe_gemm_plain<u16>(
         bf16_ptr(out), bf16_cptr(a), bf16_cptr(w), sorted_ids.data_ptr<int>(),
         expert_ids.data_ptr<int>(), n_valid.data_ptr<int>(), PM, K, N,
-        static_cast<int>(block_m), static_cast<int>(mode), current_stream());
+        static_cast<int>(block_m), static_cast<int>(mode),
+        static_cast<float>(limit), current_stream());
   else
     fi::launch_moe_gemm_plain<float>(
         out.data_ptr<float>(), a.data_ptr<float>(), w.data_ptr<float>(),
         sorted_ids.data_ptr<int>(), expert_ids.data_ptr<int>(),
         n_valid.data_ptr<int>(), PM, K, N, static_cast<int>(block_m),
-        static_cast<int>(mode), current_stream());
+        static_cast<int>(mode), static_cast<float>(limit), current_stream());
+}
+
+void moe_route_grouped(at::Tensor logits, at::Tensor correction,
+                       at::Tensor topv, at::Tensor topi, int64_t k,
+                       int64_t groups, int64_t keep) {
+  TORCH_CHECK(logits.is_cuda() && logits.scalar_type() == at::kFloat &&
+              logits.is_contiguous() && logits.dim() == 2);
+  TORCH_CHECK(correction.is_cuda() && correction.scalar_type() == at::kFloat &&
+              correction.is_contiguous());
+  TORCH_CHECK(topv.scalar_type() == at::kFloat &&
+              topi.scalar_type() == at::kInt);
+  const int T = logits.size(0);
+  const int E = logits.size(1);
+  TORCH_CHECK(correction.numel() == E);
+  TORCH_CHECK(E >= 1 && E <= 1024 && groups >= 1 && E % groups == 0 &&
+                  keep >= 1 && keep <= groups && k >= 1 &&
+                  k <= keep * (E / groups),
+              "moe_route_grouped: experts <= 1024 in equal groups, "
+              "1 <= keep <= groups, k within the kept groups");
+  TORCH_CHECK(topv.numel() == T * k && topi.numel() == T * k);
+  if (T == 0) return;
+  fi::launch_moe_route_grouped(
+      logits.data_ptr<float>(), correction.data_ptr<float>(),
+      topv.data_ptr<float>(), topi.data_ptr<int>(), T, E, (int)k, (int)groups,
+      (int)keep, current_stream());
 }
 
 void moe_route(at::Tensor logits, at::Tensor topv, at::Tensor topi, int64_t k,
@@ -256,6 +287,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "(vLLM moe_align_block_size analog)");
   m.def("moe_router_topk", &moe_router_topk,
         "fused router tail: softmax + top-k + optional renormalize");
+  m.def("moe_route_grouped", &moe_route_grouped,
+        "group-limited router tail: sigmoid scores, choice on score + "
+        "correction inside the best groups, weights = chosen scores");
   m.def("moe_route", &moe_route,
         "router tail for any expert count: softmax/sigmoid scores, top-k, "
         "renormalize, constant factor");

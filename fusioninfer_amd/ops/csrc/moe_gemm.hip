@@ -67,10 +67,12 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
     const int* __restrict__ sorted_ids, // [PM] token row per padded slot
     const int* __restrict__ expert_ids, // [PM/BM] local expert per m-tile
     const int* __restrict__ n_valid,    // device scalar: real m-tile count
-    const int K, const int N) {
+    const int K, const int N, const float limit) {
   // MODE 0: plain GEMM over act rows; 1: gathered x rows, gate|up
-  // columns, silu(gate) * up; 2: gathered x rows, up alone, relu(up)^2
-  constexpr bool GATE_UP = MODE == 1;
+  // columns, silu(gate) * up; 2: gathered x rows, up alone, relu(up)^2;
+  // 3: as 1 with the clamped unit g' sigmoid(1.702 g') (u' + 1),
+  // g' = min(g, limit), u' = clamp(u, -limit, limit)
+  constexpr bool GATE_UP = MODE == 1 || MODE == 3;
   constexpr bool GATHER = MODE != 0;
   constexpr int BM = 16 * WM * MITER;
   static_assert(!STAGE_A || BM == 128, "STAGE_A is tuned for BM=128");
@@ -255,7 +257,12 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
       for (int r = 0; r < 4; ++r) {
         const int orow = row0 + mi * 16 + (lane >> 4) * 4 + r;
         float v;
-        if (GATE_UP) {
+        if (MODE == 3) {
+          const float g = fminf(acc_g[mi][ni][r], limit);
+          const float u =
+              fminf(fmaxf(acc_u[GATE_UP ? mi : 0][ni][r], -limit), limit);
+          v = (g / (1.f + __expf(-1.702f * g))) * (u + 1.f);
+        } else if (GATE_UP) {
           const float g = acc_g[mi][ni][r];
           const float u = acc_u[mi][ni][r];
           v = (g / (1.f + __expf(-g))) * u;
@@ -486,21 +493,26 @@ __global__ __launch_bounds__(256) void moe_gemm_fp8_kernel(
 void launch_moe_gemm(u16* out, const u16* a, const u16* b,
                      const int* sorted_ids, const int* expert_ids,
                      const int* n_valid, int max_mtiles, int K, int N,
-                     int block_m, int mode, hipStream_t stream) {
+                     int block_m, int mode, float limit,
+                     hipStream_t stream) {
   if (block_m == 16) {
     const dim3 grid(max_mtiles, N / 64);
     if (mode == 1)
       hipLaunchKernelGGL((moe_gemm_kernel<1, 4, 1, 1, 1>), grid, dim3(256),
                          0, stream, out, a, b, sorted_ids, expert_ids,
-                         n_valid, K, N);
+                         n_valid, K, N, limit);
+    else if (mode == 3)
+      hipLaunchKernelGGL((moe_gemm_kernel<1, 4, 1, 1, 3>), grid, dim3(256),
+                         0, stream, out, a, b, sorted_ids, expert_ids,
+                         n_valid, K, N, limit);
     else if (mode == 2)
       hipLaunchKernelGGL((moe_gemm_kernel<1, 4, 1, 1, 2>), grid, dim3(256),
                          0, stream, out, a, b, sorted_ids, expert_ids,
-                         n_valid, K, N);
+                         n_valid, K, N, limit);
     else
       hipLaunchKernelGGL((moe_gemm_kernel<1, 4, 1, 1, 0>), grid,
                          dim3(256), 0, stream, out, a, b, sorted_ids,
-                         expert_ids, n_valid, K, N);
+                         expert_ids, n_valid, K, N, limit);
   } else {  // block_m == 128
     // FI_MOE_STAGE_A=0 falls back to the register-gather form (A/B knob)
     static const bool stage_a = [] {
@@ -512,31 +524,41 @@ void launch_moe_gemm(u16* out, const u16* a, const u16* b,
       if (stage_a)
         hipLaunchKernelGGL((moe_gemm_kernel<2, 2, 4, 2, 1, true>), grid,
                            dim3(256), 0, stream, out, a, b, sorted_ids,
-                           expert_ids, n_valid, K, N);
+                           expert_ids, n_valid, K, N, limit);
       else
         hipLaunchKernelGGL((moe_gemm_kernel<2, 2, 4, 2, 1, false>), grid,
                            dim3(256), 0, stream, out, a, b, sorted_ids,
-                           expert_ids, n_valid, K, N);
+                           expert_ids, n_valid, K, N, limit);
+    } else if (mode == 3) {
+      const dim3 grid(max_mtiles, N / 64);
+      if (stage_a)
+        hipLaunchKernelGGL((moe_gemm_kernel<2, 2, 4, 2, 3, true>), grid,
+                           dim3(256), 0, stream, out, a, b, sorted_ids,
+                           expert_ids, n_valid, K, N, limit);
+      else
+        hipLaunchKernelGGL((moe_gemm_kernel<2, 2, 4, 2, 3, false>), grid,
+                           dim3(256), 0, stream, out, a, b, sorted_ids,
+                           expert_ids, n_valid, K, N, limit);
     } else if (mode == 2) {
       const dim3 grid(max_mtiles, N / 64);
       if (stage_a)
         hipLaunchKernelGGL((moe_gemm_kernel<2, 2, 4, 2, 2, true>), grid,
                            dim3(256), 0, stream, out, a, b, sorted_ids,
-                           expert_ids, n_valid, K, N);
+                           expert_ids, n_valid, K, N, limit);
       else
         hipLaunchKernelGGL((moe_gemm_kernel<2, 2, 4, 2, 2, false>), grid,
                            dim3(256), 0, stream, out, a, b, sorted_ids,
-                           expert_ids, n_valid, K, N);
+                           expert_ids, n_valid, K, N, limit);
     } else {
       const dim3 grid(max_mtiles, N / 128);
       if (stage_a)
         hipLaunchKernelGGL((moe_gemm_kernel<2, 2, 4, 4, 0, true>), grid,
                            dim3(256), 0, stream, out, a, b, sorted_ids,
-                           expert_ids, n_valid, K, N);
+                           expert_ids, n_valid, K, N, limit);
       else
         hipLaunchKernelGGL((moe_gemm_kernel<2, 2, 4, 4, 0, false>), grid,
                            dim3(256), 0, stream, out, a, b, sorted_ids,
-                           expert_ids, n_valid, K, N);
+                           expert_ids, n_valid, K, N, limit);
     }
   }
 }

@@ -13,7 +13,15 @@
 //    operands staged through LDS as fp32. Mode 0: plain GEMM over act
 //    rows; 1: x rows gathered through sorted_ids, gate|up columns,
 //    silu(gate) * up on the way out; 2: gathered x rows, up columns
-//    alone, relu(up)^2 on the way out.
+//    alone, relu(up)^2 on the way out; 3: as 1 with the clamped unit
+//    g' sigmoid(1.702 g') (u' + 1), g' = min(g, limit),
+//    u' = clamp(u, -limit, limit).
+//  * moe_route_grouped: group-limited router tail for up to 1024 experts.
+//    One wave per token; scores s = sigmoid(z), choice scores c = s +
+//    correction. Experts form equal groups of neighbours; a group's score
+//    is the sum of its two largest choice scores, the best `keep` groups
+//    stay, and the k largest c inside them are chosen (ties: smaller
+//    index). Weights are the chosen s as they are.
 //  * moe_combine: out[t] = sum_k w[t,k] * y[pos[t,k]], any width, bf16 or
 //    fp32 rows, no atomics.
 
@@ -97,6 +105,95 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
   }
 }
 
+__global__ __launch_bounds__(256) void moe_route_grouped_kernel(
+    const float* __restrict__ logits, const float* __restrict__ correction,
+    float* __restrict__ topv, int* __restrict__ topi, const int T,
+    const int E, const int k, const int groups, const int keep) {
+  // choice scores of a token's experts, then of its groups
+  __shared__ float cs[4][1024];
+  __shared__ float gs[4][1024];
+  const int w = threadIdx.x / kWaveSize;
+  const int t = blockIdx.x * 4 + w;
+  if (t >= T) return;      // whole waves leave; no block-wide barrier below
+  const int lane = threadIdx.x % kWaveSize;
+  const float* row = logits + static_cast<int64_t>(t) * E;
+  for (int e = lane; e < E; e += 64)
+    cs[w][e] = 1.0f / (1.0f + expf(-row[e])) + correction[e];
+  __builtin_amdgcn_wave_barrier();
+  __threadfence_block();
+  if (groups > 1 && keep < groups) {
+    const int n = E / groups;
+    for (int g = lane; g < groups; g += 64) {
+      float a = -INFINITY, b = -INFINITY;     // two largest of the group
+      for (int e = g * n; e < (g + 1) * n; ++e) {
+        const float c = cs[w][e];
+        if (c > a) {
+          b = a;
+          a = c;
+        } else if (c > b) {
+          b = c;
+        }
+      }
+      gs[w][g] = n > 1 ? a + b : a;
+    }
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+    // a group stays if fewer than `keep` groups beat it (larger score, or
+    // the same score and a smaller index)
+    for (int g = lane; g < groups; g += 64) {
+      const float mine = gs[w][g];
+      int beat = 0;
+      for (int o = 0; o < groups; ++o) {
+        const float s = gs[w][o];
+        beat += (s > mine || (s == mine && o < g)) ? 1 : 0;
+      }
+      if (beat >= keep)
+        for (int e = g * n; e < (g + 1) * n; ++e) cs[w][e] = -INFINITY;
+    }
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+  }
+  float sc[kRouteSlots];
+#pragma unroll
+  for (int j = 0; j < kRouteSlots; ++j) {
+    const int e = lane + 64 * j;
+    sc[j] = e < E ? cs[w][e] : -INFINITY;
+  }
+  unsigned taken = 0;      // bit j: slot j of this lane is already chosen
+  for (int it = 0; it < k; ++it) {
+    float v = -INFINITY;
+    int idx = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < kRouteSlots; ++j) {
+      const int e = lane + 64 * j;
+      // ascending j: the smaller index wins ties
+      if (e < E && !((taken >> j) & 1u) &&
+          (idx == 0x7fffffff || sc[j] > v)) {
+        v = sc[j];
+        idx = e;
+      }
+    }
+#pragma unroll
+    for (int off = 32; off; off >>= 1) {
+      const float ov = __shfl_xor(v, off);
+      const int oi = __shfl_xor(idx, off);
+      if (oi != 0x7fffffff &&
+          (idx == 0x7fffffff || ov > v || (ov == v && oi < idx))) {
+        v = ov;
+        idx = oi;
+      }
+    }
+    if (lane == 0) {
+      topi[static_cast<int64_t>(t) * k + it] = idx;
+      topv[static_cast<int64_t>(t) * k + it] =
+          1.0f / (1.0f + expf(-row[idx]));
+    }
+#pragma unroll
+    for (int j = 0; j < kRouteSlots; ++j)
+      if (idx == lane + 64 * j) taken |= 1u << j;
+  }
+}
+
 constexpr int kPlainBM = 16;   // rows per workgroup
 constexpr int kPlainBN = 64;   // columns per workgroup
 constexpr int kPlainKT = 32;   // K step
@@ -108,8 +205,8 @@ __global__ __launch_bounds__(256) void moe_gemm_plain_kernel(
     const A* __restrict__ w,            // [E, GATE_UP ? 2N : N, K]
     const int* __restrict__ sorted_ids, const int* __restrict__ expert_ids,
     const int* __restrict__ n_valid, const int K, const int N,
-    const int block_m) {
-  constexpr bool GATE_UP = MODE == 1;
+    const int block_m, const float limit) {
+  constexpr bool GATE_UP = MODE == 1 || MODE == 3;
   constexpr bool GATHER = MODE != 0;
   // m-tiles are block_m rows; this workgroup covers 16 of them
   const int sub = block_m / kPlainBM;
@@ -169,7 +266,11 @@ __global__ __launch_bounds__(256) void moe_gemm_plain_kernel(
     const int c = col0 + cg + 16 * j;
     if (c >= N) continue;
     float v = acc[j];
-    if (GATE_UP) {
+    if (MODE == 3) {
+      const float g = fminf(acc[j], limit);
+      const float u = fminf(fmaxf(acc2[j], -limit), limit);
+      v = g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+    } else if (GATE_UP) {
       const float g = acc[j];
       v = g / (1.0f + expf(-g)) * acc2[j];
     } else if (MODE == 2) {
@@ -206,24 +307,37 @@ void launch_moe_route(const float* logits, float* topv, int* topi, int T,
                      scale);
 }
 
+void launch_moe_route_grouped(const float* logits, const float* correction,
+                              float* topv, int* topi, int T, int E, int k,
+                              int groups, int keep, hipStream_t stream) {
+  hipLaunchKernelGGL(moe_route_grouped_kernel, dim3(ceil_div(T, 4)),
+                     dim3(256), 0, stream, logits, correction, topv, topi, T,
+                     E, k, groups, keep);
+}
+
 template <typename A>
 void launch_moe_gemm_plain(A* out, const A* a, const A* w,
                            const int* sorted_ids, const int* expert_ids,
                            const int* n_valid, int PM, int K, int N,
-                           int block_m, int mode, hipStream_t stream) {
+                           int block_m, int mode, float limit,
+                           hipStream_t stream) {
   const dim3 grid(PM / kPlainBM, ceil_div(N, kPlainBN));
   if (mode == 1)
     hipLaunchKernelGGL((moe_gemm_plain_kernel<A, 1>), grid, dim3(256), 0,
                        stream, out, a, w, sorted_ids, expert_ids, n_valid, K,
-                       N, block_m);
+                       N, block_m, limit);
+  else if (mode == 3)
+    hipLaunchKernelGGL((moe_gemm_plain_kernel<A, 3>), grid, dim3(256), 0,
+                       stream, out, a, w, sorted_ids, expert_ids, n_valid, K,
+                       N, block_m, limit);
   else if (mode == 2)
     hipLaunchKernelGGL((moe_gemm_plain_kernel<A, 2>), grid, dim3(256), 0,
                        stream, out, a, w, sorted_ids, expert_ids, n_valid, K,
-                       N, block_m);
+                       N, block_m, limit);
   else
     hipLaunchKernelGGL((moe_gemm_plain_kernel<A, 0>), grid, dim3(256), 0,
                        stream, out, a, w, sorted_ids, expert_ids, n_valid, K,
-                       N, block_m);
+                       N, block_m, limit);
 }
 
 template <typename A>
@@ -237,7 +351,7 @@ void launch_moe_combine(A* out, const A* y, const int* pos, const float* w,
 #define FI_INST(A)                                                            \
   template void launch_moe_gemm_plain<A>(A*, const A*, const A*, const int*,  \
                                          const int*, const int*, int, int,    \
-                                         int, int, int, hipStream_t);         \
+                                         int, int, int, float, hipStream_t);  \
   template void launch_moe_combine<A>(A*, const A*, const int*, const float*, \
                                       int, int, int, hipStream_t);
 FI_INST(float)

@@ -133,13 +133,30 @@ bool launch_sink_attention_tiles(A*, const A*, const A*, const A*, int,
                                  const int*, int, const int*, const int*,
                                  const int*, const int*, int, const float*,
                                  const A*, int64_t, int, int, int, int, int,
-                                 float, hipStream_t);
+                                 int, float, int, int, hipStream_t);
 template <typename A>
 void launch_sink_attention_rows(A*, float*, float*, const A*, const A*,
                                 const A*, int, const int*, int, const int*,
                                 const int*, const float*, const A*, int64_t,
-                                int, int, int, int, int, int, int, float, int,
-                                hipStream_t);
+                                int, int, int, int, int, int, int, int, float,
+                                int, int, int, hipStream_t);
+template <typename A>
+void launch_pair_embed(float*, A*, const int64_t*, const A*, float, const A*,
+                       int64_t, int64_t, int64_t, int*, const int*,
+                       const int*, const int*, const int*, int, int,
+                       hipStream_t);
+template <typename I, typename A>
+void launch_norm_affine(const I*, float*, A*, const float*, const float*,
+                        float, int, int, hipStream_t);
+template <typename A>
+void launch_widenorm_rope_cache(A*, const A*, int64_t, const A*, int64_t,
+                                const A*, int64_t, const int*, const float*,
+                                const float*, float, const float*, int, float,
+                                A*, A*, const int*, int, int, int, int, int,
+                                int, hipStream_t);
+template <typename A>
+void launch_clamped_glu(A*, const A*, int64_t, int, int, float, hipStream_t);
+void launch_tanh_cap(float*, int64_t, float, hipStream_t);
 
 }  // namespace fi
 
@@ -913,9 +930,11 @@ void sink_paged_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
                           c10::optional<at::Tensor> tile_row0,
                           int64_t tile_rows,
                           c10::optional<at::Tensor> part_ml,
-                          c10::optional<at::Tensor> part_o) {
+                          c10::optional<at::Tensor> part_o, int64_t window,
+                          int64_t keep_first) {
   CHECK_ACT(q);
   CHECK_ACT(out);
+  TORCH_CHECK(window >= 0 && keep_first >= 0);
   CHECK_I32(row_seq);
   CHECK_I32(positions);
   TORCH_CHECK(seq_bt.is_cuda() && seq_bt.scalar_type() == at::kInt &&
@@ -953,9 +972,11 @@ void sink_paged_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
   }
   const void* gp = nullptr;
   int64_t g_stride = 0;
+  int gate_elem = 0;   // 1: one gate per entry [T, H*DV], 0: per head [T, H]
   if (gate.has_value()) {
     TORCH_CHECK(gate->is_cuda() && gate->scalar_type() == dt);
-    check_rows(*gate, T, H, "output gate");
+    gate_elem = gate->dim() == 2 && gate->size(1) == H * DV && DV > 1;
+    check_rows(*gate, T, gate_elem ? H * DV : H, "output gate");
     gp = gate->data_ptr();
     g_stride = gate->stride(0);
   }
@@ -977,8 +998,9 @@ void sink_paged_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
                       seq_cu->data_ptr<int>(), positions.data_ptr<int>(),
                       tile_seq->data_ptr<int>(), tile_row0->data_ptr<int>(),
                       (int)tile_seq->numel(), sp,
-                      reinterpret_cast<const A*>(gp), g_stride, H, G, DK,
-                      (int)DV, bs, (float)scale, stream()));
+                      reinterpret_cast<const A*>(gp), g_stride, gate_elem, H,
+                      G, DK, (int)DV, bs, (float)scale, (int)window,
+                      (int)keep_first, stream()));
     if (ok) done = tile_rows;
   }
   if (done == T) return;
@@ -1001,8 +1023,9 @@ void sink_paged_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
                         reinterpret_cast<const A*>(vp), v_row,
                         seq_bt.data_ptr<int>(), (int)seq_bt.stride(0),
                         row_seq.data_ptr<int>(), positions.data_ptr<int>(),
-                        sp, reinterpret_cast<const A*>(gp), g_stride, row0,
-                        rows, H, G, DK, (int)DV, bs, (float)scale, ns,
+                        sp, reinterpret_cast<const A*>(gp), g_stride,
+                        gate_elem, row0, rows, H, G, DK, (int)DV, bs,
+                        (float)scale, ns, (int)window, (int)keep_first,
                         stream()));
   }
 }
@@ -1126,7 +1149,196 @@ void relu_squared(at::Tensor out, at::Tensor x) {
                                              (int)x.size(1), stream()));
 }
 
+void pair_embed(at::Tensor resid, at::Tensor act, at::Tensor ids,
+                at::Tensor embed, double scale,
+                c10::optional<at::Tensor> pair_table, int64_t buckets,
+                int64_t mul_prev, int64_t mul_cur, at::Tensor prev_token,
+                at::Tensor seq_cu, at::Tensor row_seq, at::Tensor seq_slots,
+                at::Tensor positions) {
+  CHECK_F32(resid);
+  CHECK_ACT(embed);
+  CHECK_I32(prev_token);
+  CHECK_I32(seq_cu);
+  CHECK_I32(row_seq);
+  CHECK_I32(seq_slots);
+  CHECK_I32(positions);
+  TORCH_CHECK(ids.is_cuda() && ids.scalar_type() == at::kLong &&
+              ids.is_contiguous());
+  const int64_t T = ids.numel();
+  TORCH_CHECK(embed.dim() == 2 && embed.is_contiguous());
+  const int64_t W = embed.size(1);
+  const auto dt = embed.scalar_type();
+  TORCH_CHECK(resid.is_contiguous() && resid.numel() == T * W);
+  TORCH_CHECK(act.is_cuda() && act.is_contiguous() &&
+              act.scalar_type() == dt && act.numel() == T * W);
+  TORCH_CHECK(row_seq.numel() == T && positions.numel() == T);
+  TORCH_CHECK(seq_cu.numel() >= 1 && seq_slots.numel() >= seq_cu.numel() - 1);
+  TORCH_CHECK(buckets >= 1);
+  const void* pt = nullptr;
+  if (pair_table.has_value()) {
+    TORCH_CHECK(pair_table->is_cuda() && pair_table->is_contiguous() &&
+                pair_table->scalar_type() == dt && pair_table->dim() == 2 &&
+                pair_table->size(0) == buckets + 1 &&
+                pair_table->size(1) == W);
+    pt = pair_table->data_ptr();
+  }
+  DISPATCH_ACT(embed, fi::launch_pair_embed<A>(
+                          resid.data_ptr<float>(), ptr<A>(act),
+                          ids.data_ptr<int64_t>(), ptr<A>(embed), (float)scale,
+                          reinterpret_cast<const A*>(pt), buckets, mul_prev,
+                          mul_cur, prev_token.data_ptr<int>(),
+                          seq_cu.data_ptr<int>(), row_seq.data_ptr<int>(),
+                          seq_slots.data_ptr<int>(), positions.data_ptr<int>(),
+                          (int)T, (int)W, stream()));
+}
+
+void layer_norm_affine(at::Tensor out, at::Tensor x, at::Tensor w,
+                       at::Tensor b, double eps) {
+  CHECK_F32(x);
+  CHECK_ACT(out);
+  CHECK_F32(w);
+  CHECK_F32(b);
+  TORCH_CHECK(x.dim() == 2 && x.is_contiguous() && out.is_contiguous() &&
+              out.sizes() == x.sizes());
+  const int T = x.size(0), W = x.size(1);
+  TORCH_CHECK(w.numel() == W && b.numel() == W);
+  if (out.scalar_type() == at::kFloat)
+    fi::launch_norm_affine<float, float>(
+        x.data_ptr<float>(), nullptr, out.data_ptr<float>(),
+        w.data_ptr<float>(), b.data_ptr<float>(), (float)eps, T, W, stream());
+  else
+    fi::launch_norm_affine<float, fi::u16>(
+        x.data_ptr<float>(), nullptr, ptr<fi::u16>(out), w.data_ptr<float>(),
+        b.data_ptr<float>(), (float)eps, T, W, stream());
+}
+
+// resid += layer_norm(y) * w + b; out (activation dtype) = rounded resid.
+// For fp32 activations out is resid itself.
+void post_norm_residual(at::Tensor resid, at::Tensor y, at::Tensor w,
+                        at::Tensor b, at::Tensor out, double eps) {
+  CHECK_F32(resid);
+  CHECK_ACT(y);
+  CHECK_F32(w);
+  CHECK_F32(b);
+  TORCH_CHECK(resid.dim() == 2 && resid.is_contiguous() &&
+              y.is_contiguous() && y.sizes() == resid.sizes());
+  const int T = resid.size(0), W = resid.size(1);
+  TORCH_CHECK(w.numel() == W && b.numel() == W);
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() &&
+              out.scalar_type() == y.scalar_type() &&
+              out.sizes() == resid.sizes());
+  if (y.scalar_type() == at::kFloat) {
+    TORCH_CHECK(out.data_ptr() == resid.data_ptr(),
+                "fp32 activations read the stream itself");
+    fi::launch_norm_affine<float, float>(
+        y.data_ptr<float>(), resid.data_ptr<float>(), nullptr,
+        w.data_ptr<float>(), b.data_ptr<float>(), (float)eps, T, W, stream());
+  } else {
+    fi::launch_norm_affine<fi::u16, fi::u16>(
+        ptr<fi::u16>(y), resid.data_ptr<float>(), ptr<fi::u16>(out),
+        w.data_ptr<float>(), b.data_ptr<float>(), (float)eps, T, W, stream());
+  }
+}
+
+void widenorm_rope_cache(at::Tensor q_out, at::Tensor q,
+                         c10::optional<at::Tensor> k,
+                         c10::optional<at::Tensor> v, at::Tensor positions,
+                         at::Tensor q_w, c10::optional<at::Tensor> k_w,
+                         double eps, at::Tensor inv_freq, double rot_mult,
+                         at::Tensor k_cache, at::Tensor v_cache,
+                         at::Tensor slot_mapping, int64_t H, int64_t G,
+                         int64_t D, int64_t V) {
+  CHECK_ACT(q);
+  CHECK_ACT(q_out);
+  CHECK_I32(positions);
+  CHECK_I32(slot_mapping);
+  CHECK_F32(q_w);
+  CHECK_F32(inv_freq);
+  const int64_t T = q.size(0);
+  check_rows(q, T, H * D, "q");
+  const auto dt = q.scalar_type();
+  TORCH_CHECK(q_out.scalar_type() == dt && q_out.is_contiguous() &&
+              q_out.numel() == T * H * D);
+  TORCH_CHECK(positions.numel() == T && slot_mapping.numel() == T);
+  TORCH_CHECK(q_w.numel() == H * D);
+  const int nrot = 2 * (int)inv_freq.numel();
+  TORCH_CHECK(nrot <= D, "more turning pairs than the head holds");
+  TORCH_CHECK(H >= 1 && G >= 1 && D >= 1 && V >= 1);
+  const void *kp = nullptr, *vp = nullptr;
+  const float* kw = nullptr;
+  int64_t ks = 0, vs = 0;
+  void *kc = nullptr, *vc = nullptr;
+  int bs = 1;
+  if (k.has_value()) {
+    TORCH_CHECK(v.has_value() && k_w.has_value());
+    CHECK_ACT(*k);
+    CHECK_ACT(*v);
+    CHECK_F32(*k_w);
+    check_rows(*k, T, G * D, "k");
+    check_rows(*v, T, G * V, "v");
+    TORCH_CHECK(k->scalar_type() == dt && v->scalar_type() == dt);
+    TORCH_CHECK(k_w->numel() == G * D);
+    TORCH_CHECK(k_cache.is_cuda() && v_cache.is_cuda() &&
+                k_cache.is_contiguous() && v_cache.is_contiguous() &&
+                k_cache.scalar_type() == dt && v_cache.scalar_type() == dt);
+    TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 &&
+                k_cache.size(0) == v_cache.size(0) && k_cache.size(1) == G &&
+                v_cache.size(1) == G && k_cache.size(2) == v_cache.size(2) &&
+                k_cache.size(3) == D && v_cache.size(3) == V);
+    kp = k->data_ptr();
+    vp = v->data_ptr();
+    kw = k_w->data_ptr<float>();
+    ks = k->stride(0);
+    vs = v->stride(0);
+    kc = k_cache.data_ptr();
+    vc = v_cache.data_ptr();
+    bs = k_cache.size(2);
+  }
+  DISPATCH_ACT(q, fi::launch_widenorm_rope_cache<A>(
+                      ptr<A>(q_out), ptr<A>(q), q.stride(0),
+                      reinterpret_cast<const A*>(kp), ks,
+                      reinterpret_cast<const A*>(vp), vs,
+                      positions.data_ptr<int>(), q_w.data_ptr<float>(), kw,
+                      (float)eps, inv_freq.data_ptr<float>(), nrot,
+                      (float)rot_mult, reinterpret_cast<A*>(kc),
+                      reinterpret_cast<A*>(vc), slot_mapping.data_ptr<int>(),
+                      (int)T, (int)H, (int)G, (int)D, (int)V, bs, stream()));
+}
+
+void clamped_glu(at::Tensor out, at::Tensor gu, double limit) {
+  CHECK_ACT(gu);
+  CHECK_ACT(out);
+  TORCH_CHECK(gu.dim() == 2 && gu.stride(1) == 1 && gu.size(1) % 2 == 0);
+  const int T = gu.size(0), F = gu.size(1) / 2;
+  TORCH_CHECK(out.is_contiguous() && out.scalar_type() == gu.scalar_type() &&
+              out.dim() == 2 && out.size(0) == T && out.size(1) == F);
+  DISPATCH_ACT(gu, fi::launch_clamped_glu<A>(ptr<A>(out), ptr<A>(gu),
+                                             gu.stride(0), T, F, (float)limit,
+                                             stream()));
+}
+
+void tanh_cap(at::Tensor x, double cap) {
+  CHECK_F32(x);
+  TORCH_CHECK(x.is_contiguous() && cap > 0);
+  fi::launch_tanh_cap(x.data_ptr<float>(), x.numel(), (float)cap, stream());
+}
+
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("pair_embed", &pair_embed,
+        "embedding times a constant plus a (previous id, id) table row; the "
+        "previous id of a group's first row lives in a slot state");
+  m.def("layer_norm_affine", &layer_norm_affine,
+        "layer norm with weight and bias of fp32 rows");
+  m.def("post_norm_residual", &post_norm_residual,
+        "stream += layer_norm(sublayer output) * w + b, emits the rounded "
+        "stream");
+  m.def("widenorm_rope_cache", &widenorm_rope_cache,
+        "whole-projection RMS norm of q/k, interleaved partial rotation "
+        "with given frequencies, k and v into the paged caches");
+  m.def("clamped_glu", &clamped_glu,
+        "min(g, L) sigmoid(1.702 min(g, L)) (clamp(u, -L, L) + 1)");
+  m.def("tanh_cap", &tanh_cap, "x <- cap tanh(x / cap), fp32 in place");
   m.def("scaled_residual_layer_norm", &scaled_residual_layer_norm,
         "fp32 stream += scaled sublayer results, then layer norm");
   m.def("headnorm_qtemp_cache", &headnorm_qtemp_cache,

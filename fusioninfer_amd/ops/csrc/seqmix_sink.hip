@@ -1,7 +1,10 @@
 // Causal softmax attention over the paged cache with separate key and
 // value sizes, an optional per-head sink in the denominator, values that
-// may be a leading slice of the cached key rows, and an optional sigmoid
-// gate per (row, head) on the result.
+// may be a leading slice of the cached key rows, an optional sigmoid gate
+// on the result (per (row, head), or per entry), and an optional sliding
+// window that keeps the first keys: with window > 0 position p sees key j
+// only if p - j < window or j < keep_first. Tiles and spans that no row
+// can see are skipped.
 //
 //  * split form (any sizes): a workgroup takes one row, a batch of up to
 //    8 query heads that share a key/value head, and one span of 256 keys:
@@ -32,6 +35,16 @@ namespace {
 constexpr int kSpanKeys = 256;   // keys per workgroup of the split form
 constexpr int kHeadBatch = 8;    // query heads per workgroup
 
+FI_DEV bool key_visible(int p, int j, int window, int keep_first) {
+  return j <= p && (window <= 0 || p - j < window || j < keep_first);
+}
+
+// a 256-key span holds at least one key that position p sees
+FI_DEV bool span_live(int p, int j0, int window, int keep_first) {
+  return j0 <= p && (window <= 0 || j0 < keep_first ||
+                     j0 + kSpanKeys > p - window + 1);
+}
+
 template <typename A, int VW>
 __global__ __launch_bounds__(256) void sink_attention_split_kernel(
     float* __restrict__ part_ml,      // [rows, H, ns, 2]
@@ -41,7 +54,7 @@ __global__ __launch_bounds__(256) void sink_attention_split_kernel(
     const int* __restrict__ seq_bt, int bt_stride,
     const int* __restrict__ row_seq, const int* __restrict__ positions,
     int row0, int H, int G, int DK, int DV, int dv_round, int bs, float scale,
-    int ns, int hb, int tpr) {
+    int ns, int hb, int tpr, int window, int keep_first) {
   extern __shared__ float smem[];
   float* qs = smem;                               // [kHeadBatch][DK]
   float* ps = qs + kHeadBatch * DK;               // [kHeadBatch][256]
@@ -61,7 +74,8 @@ __global__ __launch_bounds__(256) void sink_attention_split_kernel(
   const int span = blockIdx.z;
   const int p = positions[t];
   const int j0 = span * kSpanKeys;
-  if (j0 > p) return;                 // the combine step never reads it
+  // the combine step never reads a span that is not live
+  if (!span_live(p, j0, window, keep_first)) return;
   const int nkeys = min(kSpanKeys, p - j0 + 1);
 
   const A* qp = q + (static_cast<int64_t>(t) * H + h0) * DK;
@@ -70,15 +84,20 @@ __global__ __launch_bounds__(256) void sink_attention_split_kernel(
   __syncthreads();
 
   const int* bt = seq_bt + static_cast<int64_t>(row_seq[t]) * bt_stride;
-  const bool valid = tid < nkeys;
+  // keys outside the window keep a weight of zero; their value rows are
+  // still addressed (they stay in the sequence's pages)
+  const bool valid =
+      tid < nkeys && key_visible(p, j0 + tid, window, keep_first);
   float dots[kHeadBatch];
 #pragma unroll
   for (int i = 0; i < kHeadBatch; ++i) dots[i] = 0.f;
-  if (valid) {
+  int64_t rowi = 0;
+  if (tid < nkeys) {
     const int j = j0 + tid;
-    const int64_t rowi =
-        (static_cast<int64_t>(bt[j / bs]) * G + g) * bs + j % bs;
+    rowi = (static_cast<int64_t>(bt[j / bs]) * G + g) * bs + j % bs;
     voff[tid] = rowi * v_row;
+  }
+  if (valid) {
     const A* kp = k_cache + rowi * DK;
     for (int d0 = 0; d0 < DK; d0 += VW) {
       float kv[VW];
@@ -214,27 +233,46 @@ __global__ __launch_bounds__(64) void sink_attention_combine_kernel(
     A* __restrict__ out,              // [T, H, DV]
     const float* __restrict__ part_ml, const float* __restrict__ part_o,
     const int* __restrict__ positions, const float* __restrict__ sink,
-    const A* __restrict__ gate, int64_t g_stride, int row0, int H, int DV,
-    int ns) {
+    const A* __restrict__ gate, int64_t g_stride, int gate_elem, int row0,
+    int H, int DV, int ns, int window, int keep_first) {
   const int r = blockIdx.x, h = blockIdx.y;
   const int t = row0 + r;
   const int lane = threadIdx.x;
-  const int nsp = positions[t] / kSpanKeys + 1;
+  const int p = positions[t];
+  const int nsp = p / kSpanKeys + 1;
+  // with a window the live spans are those of the kept first keys and
+  // those that reach into the window
+  int s_win = 0, s_keep = nsp;
+  if (window > 0) {
+    s_win = max(p - window + 1, 0) / kSpanKeys;
+    s_keep = min(s_win, (keep_first + kSpanKeys - 1) / kSpanKeys);
+  }
   const float* ml = part_ml + (static_cast<int64_t>(r) * H + h) * ns * 2;
   const float* po = part_o + (static_cast<int64_t>(r) * H + h) * ns * DV;
+  auto live = [&](int s) { return s < s_keep || s >= s_win; };
   float m = sink != nullptr ? sink[h] : -INFINITY;
-  for (int s = 0; s < nsp; ++s) m = fmaxf(m, ml[2 * s]);
+  for (int s = 0; s < nsp; ++s)
+    if (live(s)) m = fmaxf(m, ml[2 * s]);
   float l = sink != nullptr ? expf(sink[h] - m) : 0.f;
-  for (int s = 0; s < nsp; ++s) l += ml[2 * s + 1] * expf(ml[2 * s] - m);
+  for (int s = 0; s < nsp; ++s)
+    if (live(s)) l += ml[2 * s + 1] * expf(ml[2 * s] - m);
   float f = 1.0f / l;
-  if (gate != nullptr)
-    f *= sigmoidf_acc(Act<A>::ld(gate + t * g_stride + h));
+  const A* gp = nullptr;
+  if (gate != nullptr) {
+    if (gate_elem)
+      gp = gate + t * g_stride + static_cast<int64_t>(h) * DV;
+    else
+      f *= sigmoidf_acc(Act<A>::ld(gate + t * g_stride + h));
+  }
   A* op = out + (static_cast<int64_t>(t) * H + h) * DV;
   for (int d = lane; d < DV; d += 64) {
     float acc = 0.f;
     for (int s = 0; s < nsp; ++s)
-      acc += po[static_cast<int64_t>(s) * DV + d] * expf(ml[2 * s] - m);
-    Act<A>::st(op + d, acc * f);
+      if (live(s))
+        acc += po[static_cast<int64_t>(s) * DV + d] * expf(ml[2 * s] - m);
+    acc *= f;
+    if (gp != nullptr) acc *= sigmoidf_acc(Act<A>::ld(gp + d));
+    Act<A>::st(op + d, acc);
   }
 }
 
@@ -250,7 +288,8 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
     const int* __restrict__ seq_cu, const int* __restrict__ positions,
     const int* __restrict__ tile_seq, const int* __restrict__ tile_row0,
     const float* __restrict__ sink, const A* __restrict__ gate,
-    int64_t g_stride, int H, int G, int block_size, float scale) {
+    int64_t g_stride, int gate_elem, int H, int G, int block_size,
+    float scale, int window, int keep_first) {
   constexpr bool BF = std::is_same<A, u16>::value;
   constexpr int VEC = BF ? 8 : 4;               // elements per 16-byte load
   constexpr int KP = DK + (BF ? 8 : 4);         // K tile [BN][KP]
@@ -328,7 +367,18 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
   };
   const int wave_rows = min(16 * QS, nrows - wave * 16 * QS);
   const int wave_min_pos = wave_rows > 0 ? p_first + wave * 16 * QS : -1;
+  const int wave_max_pos = wave_min_pos + wave_rows - 1;
   const bool wave_full = wave_rows == 16 * QS;
+  // key tiles nobody in the workgroup sees lie between the kept first keys
+  // and the window of the first row (the one that reaches back farthest)
+  const int skip_lo = ((keep_first + BN - 1) / BN) * BN;
+  const int skip_hi =
+      window > 0 ? (max(p_first - window + 1, 0) / BN) * BN : 0;
+  auto next_tile = [&](int j0) {
+    const int j = j0 + BN;
+    return (j >= skip_lo && j < skip_hi) ? skip_hi : j;
+  };
+  const int j_start = (skip_lo == 0 && skip_hi > 0) ? skip_hi : 0;
 
   // K and V tiles travel global -> registers -> LDS. With PF (the large
   // sizes, whose register budget is spent anyway) the loads of the NEXT
@@ -423,17 +473,19 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
     }
   };
 
-  if constexpr (PF) load_tile(0);
-  for (int j0 = 0; j0 <= kv_hi; j0 += BN) {
+  if constexpr (PF) load_tile(j_start);
+  for (int j0 = j_start; j0 <= kv_hi; j0 = next_tile(j0)) {
     if constexpr (!PF) load_tile(j0);
     store_tile();
     __syncthreads();
     if constexpr (PF) {
-      if (j0 + BN <= kv_hi) load_tile(j0 + BN);
+      if (next_tile(j0) <= kv_hi) load_tile(next_tile(j0));
     }
 
     // ---- S^T = K Q^T ----
-    const bool interior = wave_full && j0 + BN - 1 <= wave_min_pos;
+    const bool interior =
+        wave_full && j0 + BN - 1 <= wave_min_pos &&
+        (window <= 0 || wave_max_pos - j0 < window || j0 + BN <= keep_first);
     float sv[NQ][NB][4];
     float tmax[NQ];
 #pragma unroll
@@ -469,7 +521,8 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int key = j0 + nb * 16 + 4 * g4 + i;
-          const bool vis = interior || key <= my_pos[qs];
+          const bool vis =
+              interior || key_visible(my_pos[qs], key, window, keep_first);
           sv[qs][nb][i] = vis ? acc[qs][i] * sc : -INFINITY;
           tmax[qs] = fmaxf(tmax[qs], sv[qs][nb][i]);
         }
@@ -558,14 +611,23 @@ __global__ __launch_bounds__(256) void sink_attention_tile_kernel(
     }
     float f = 1.0f / lt;
     const int64_t row = row_first + my_row[qs];
-    if (gate != nullptr)
-      f *= sigmoidf_acc(Act<A>::ld(gate + row * g_stride + h));
+    const A* gp = nullptr;
+    if (gate != nullptr) {
+      if (gate_elem)
+        gp = gate + row * g_stride + static_cast<int64_t>(h) * DV;
+      else
+        f *= sigmoidf_acc(Act<A>::ld(gate + row * g_stride + h));
+    }
     A* op = out + (row * H + h) * DV;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        Act<A>::st(op + db * 16 + 4 * g4 + i, o[qs][db][i] * f);
+      for (int i = 0; i < 4; ++i) {
+        const int d = db * 16 + 4 * g4 + i;
+        float val = o[qs][db][i] * f;
+        if (gp != nullptr) val *= sigmoidf_acc(Act<A>::ld(gp + d));
+        Act<A>::st(op + d, val);
+      }
   }
 }
 
@@ -590,9 +652,10 @@ bool launch_sink_attention_tiles(A* out, const A* q, const A* k_cache,
                                  const int* seq_cu, const int* positions,
                                  const int* tile_seq, const int* tile_row0,
                                  int num_tiles, const float* sink,
-                                 const A* gate, int64_t g_stride, int H, int G,
-                                 int DK, int DV, int block_size, float scale,
-                                 hipStream_t s) {
+                                 const A* gate, int64_t g_stride,
+                                 int gate_elem, int H, int G, int DK, int DV,
+                                 int block_size, float scale, int window,
+                                 int keep_first, hipStream_t s) {
   constexpr bool BF = std::is_same<A, u16>::value;
   if (num_tiles == 0) return true;
   // head pairs (HP_ == 2) need an even number of heads per key/value head
@@ -603,7 +666,8 @@ bool launch_sink_attention_tiles(A* out, const A* q, const A* k_cache,
         (sink_attention_tile_kernel<A, K_, V_, (BF ? BNB : BNF), QS_, HP_>),   \
         dim3(num_tiles, H / HP_, 2 / QS_), dim3(256), 0, s, out, q, k_cache,   \
         v_cache, v_row, seq_bt, bt_stride, seq_cu, positions, tile_seq,        \
-        tile_row0, sink, gate, g_stride, H, G, block_size, scale);             \
+        tile_row0, sink, gate, g_stride, gate_elem, H, G, block_size, scale,   \
+        window, keep_first);                                                   \
     return true;                                                               \
   }
   FI_TILE(64, 64, 64, 64, 2, 1)
@@ -623,9 +687,10 @@ void launch_sink_attention_rows(A* out, float* part_ml, float* part_o,
                                 const int* seq_bt, int bt_stride,
                                 const int* row_seq, const int* positions,
                                 const float* sink, const A* gate,
-                                int64_t g_stride, int row0, int rows, int H,
-                                int G, int DK, int DV, int block_size,
-                                float scale, int ns, hipStream_t s) {
+                                int64_t g_stride, int gate_elem, int row0,
+                                int rows, int H, int G, int DK, int DV,
+                                int block_size, float scale, int ns,
+                                int window, int keep_first, hipStream_t s) {
   if (rows == 0) return;
   const int rep = H / G;
   const int hb = min(kHeadBatch, rep);
@@ -659,7 +724,8 @@ void launch_sink_attention_rows(A* out, float* part_ml, float* part_o,
   hipLaunchKernelGGL((sink_attention_split_kernel<A, VW_>), grid, dim3(256),   \
                      lds, s, part_ml, part_o, q, k_cache, v_cache, v_row,      \
                      seq_bt, bt_stride, row_seq, positions, row0, H, G, DK,    \
-                     DV, dv_round, block_size, scale, ns, hb, tpr)
+                     DV, dv_round, block_size, scale, ns, hb, tpr, window,     \
+                     keep_first)
   if constexpr (BF) {
     if (vw == 8) FI_SPLIT(8);
     else if (vw == 4) FI_SPLIT(4);
@@ -671,18 +737,18 @@ void launch_sink_attention_rows(A* out, float* part_ml, float* part_o,
 #undef FI_SPLIT
   hipLaunchKernelGGL(sink_attention_combine_kernel<A>, dim3(rows, H), dim3(64),
                      0, s, out, part_ml, part_o, positions, sink, gate,
-                     g_stride, row0, H, DV, ns);
+                     g_stride, gate_elem, row0, H, DV, ns, window, keep_first);
 }
 
 #define FI_INST(A)                                                             \
   template bool launch_sink_attention_tiles<A>(                                \
       A*, const A*, const A*, const A*, int, const int*, int, const int*,      \
       const int*, const int*, const int*, int, const float*, const A*,         \
-      int64_t, int, int, int, int, int, float, hipStream_t);                   \
+      int64_t, int, int, int, int, int, int, float, int, int, hipStream_t);    \
   template void launch_sink_attention_rows<A>(                                 \
       A*, float*, float*, const A*, const A*, const A*, int, const int*, int,  \
       const int*, const int*, const float*, const A*, int64_t, int, int, int,  \
-      int, int, int, int, float, int, hipStream_t);
+      int, int, int, int, int, float, int, int, int, hipStream_t);
 FI_INST(float)
 FI_INST(u16)
 #undef FI_INST

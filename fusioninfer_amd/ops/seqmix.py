@@ -517,8 +517,8 @@ blended_rotary = ref.blended_rotary
 
 
 def pair_embed(ids, embed, embed_scale: float, pair_table, buckets: int,
-               mul_prev: int, mul_cur: int, prev_token, seq_cu, seq_slots,
-               positions, act_dtype):
+               mul_prev: int, mul_cur: int, prev_token, seq_cu, row_seq,
+               seq_slots, positions, act_dtype):
     """Start of an fp32 stream: embed[id] * embed_scale plus the pair
     table's row for (previous id, id) (row ``buckets`` at position 0). The
     previous id of a group's first row is read from ``prev_token`` [slots]
@@ -531,8 +531,8 @@ def pair_embed(ids, embed, embed_scale: float, pair_table, buckets: int,
                torch.empty((T, W), dtype=act_dtype, device=embed.device))
         _native().pair_embed(resid, act, ids, embed, float(embed_scale),
                              pair_table, int(buckets), int(mul_prev),
-                             int(mul_cur), prev_token, seq_cu, seq_slots,
-                             positions)
+                             int(mul_cur), prev_token, seq_cu, row_seq,
+                             seq_slots, positions)
         return resid, act
     return ref.pair_embed(ids, embed, embed_scale, pair_table, buckets,
                           mul_prev, mul_cur, prev_token, seq_cu, seq_slots,
