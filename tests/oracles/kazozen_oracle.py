@@ -111,29 +111,43 @@ def keys_values(h, W, pre, m, eps, pos0=0):
     return ks, v.reshape(-1, G, V)
 
 
-def attention_mixer(h, W, pre, m, eps, kv, pos0=0):
-    """h: rows at positions pos0..; kv = (keys, values) of positions 0..
-    (the layer's own or the borrowed ones). Returns the projected output."""
-    H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    T = h.shape[0]
+def attend_row(q, ks, vs, p, mask, scale, sinks):
+    """One query row q [H, D] at position p over keys ks [>=p+1, G, D] and
+    values vs [>=p+1, G, V]; returns [H, V]."""
+    H, G = q.shape[0], ks.shape[1]
+    js = [j for j in range(p + 1) if sees(p, j, mask)]
+    out = []
+    for hh in range(H):
+        g = hh // (H // G)
+        sc = (ks[js, g] @ q[hh]) * scale
+        top = torch.maximum(sc.max(), sinks[hh])
+        ex = torch.exp(sc - top)
+        den = ex.sum() + torch.exp(sinks[hh] - top)
+        out.append((ex / den) @ vs[js, g])
+    return torch.stack(out)
+
+
+def queries(h, W, pre, m, eps, pos0=0):
+    """Normed, rotated queries [T, H, dim] of rows h at positions pos0.."""
+    H, D = m["heads"], m["dim"]
     q = h @ W[pre + "q"].T + W[pre + "q.b"]
     q = unit_rms(q, eps) * W[pre + "q.norm"]
     freqs, mult = rotary_frequencies(m["rot"]) if m.get("rot") else ([], 1.0)
+    return torch.stack([rotate_interleaved(q[t].reshape(H, D), pos0 + t,
+                                           freqs, mult)
+                        for t in range(h.shape[0])])
+
+
+def attention_mixer(h, W, pre, m, eps, kv, pos0=0):
+    """h: rows at positions pos0..; kv = (keys, values) of positions 0..
+    (the layer's own or the borrowed ones). Returns the projected output."""
+    T = h.shape[0]
+    q = queries(h, W, pre, m, eps, pos0)
     gate = torch.sigmoid(h @ W[pre + "g"].T)
     ks, vs = kv
-    out = torch.zeros(T, H * V, dtype=F64)
-    for t in range(T):
-        p = pos0 + t
-        qt = rotate_interleaved(q[t].reshape(H, D), p, freqs, mult)
-        for hh in range(H):
-            g = hh // (H // G)
-            js = [j for j in range(p + 1) if sees(p, j, m.get("mask"))]
-            sc = (ks[js, g] @ qt[hh]) * m["scale"]
-            sink = W[pre + "sink"][hh]
-            top = torch.maximum(sc.max(), sink)
-            ex = torch.exp(sc - top)
-            den = ex.sum() + torch.exp(sink - top)
-            out[t, hh * V:(hh + 1) * V] = (ex / den) @ vs[js, g]
+    out = torch.stack([
+        attend_row(q[t], ks, vs, pos0 + t, m.get("mask"), m["scale"],
+                   W[pre + "sink"]).reshape(-1) for t in range(T)])
     return (out * gate) @ W[pre + "o"].T
 
 
@@ -211,3 +225,10 @@ def forward(tokens, W, cfg, trace=None):
     if cap:
         logits = cap * torch.tanh(logits / cap)
     return logits
+
+
+def greedy(prompt, W, cfg, n_new):
+    toks = list(prompt)
+    for _ in range(n_new):
+        toks.append(int(forward(toks, W, cfg)[-1].argmax()))
+    return toks[len(prompt):]
