@@ -72,22 +72,23 @@ def parse_args():
                         "workload mode; headline stays spec-off)")
     p.add_argument("--mixer-compare", action="store_true",
                    help="instead of the serving benchmark: prefill and "
-                        "decode token throughput of the Momedra, Sefalorn and "
-                        "Pinuvik designs at real-model layer sizes (random "
+                        "decode token throughput of the Kazozen, Momedra, "
+                        "Sefalorn and Pinuvik designs at real-model layer "
+                        "sizes (random "
                         "weights) next to the Qwen3-style transformer of "
                         "the same sizes")
     p.add_argument("--mc-sizes", default="2048x16,4096x32",
                    help="WIDTHxHEADS list for --mixer-compare (head dim "
                         "128, kv heads = heads/4, ff = 3*width)")
     p.add_argument("--mc-archs",
-                   default="momedra,sefalorn,pinuvik,transformer")
+                   default="kazozen,momedra,sefalorn,pinuvik,transformer")
     p.add_argument("--mc-layers", type=int, default=4)
     p.add_argument("--mc-prompt", type=int, default=2048)
     p.add_argument("--mc-prefill-seqs", type=int, default=4)
     p.add_argument("--mc-decode-batch", type=int, default=64)
     p.add_argument("--mc-chunk", type=int, default=1024,
                    help="attention chunk / window (mask size) of the "
-                        "Pinuvik and Sefalorn layers")
+                        "Pinuvik, Sefalorn and Kazozen layers")
     return p.parse_args()
 
 
@@ -104,6 +105,41 @@ def _mixer_compare_config(arch, width, heads, layers, chunk, vocab=32000):
         mc.hidden_size, mc.num_layers = width, layers
         mc.num_heads, mc.num_kv_heads, mc.head_dim = heads, kv, dim
         mc.intermediate_size, mc.vocab_size = ff, vocab
+        return mc
+    if arch == "kazozen":
+        # windowed sink attention with 4 kept first keys; every second
+        # layer reads the keys and values of the layer before it; dense
+        # and routed feed-forwards alternate, the routed ones' active size
+        # (top * ff) equals the dense ff
+        rot = {"dims": dim, "base": 1e6,
+               "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0,
+                           "slow": 1.0}}
+
+        def mixer(src=None):
+            m = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim,
+                 "scale": dim ** -0.5, "rot": rot,
+                 "mask": {"size": chunk, "keep_first": 4}}
+            if src is not None:
+                m["kv_from"] = src
+            return m
+
+        moe = {"kind": "moe", "expert": {"ff": ff // 2, "limit": 7.0},
+               "router": {"experts": 8, "top": 2,
+                          "groups": {"count": 4, "keep": 2}}}
+        dense = {"kind": "dense", "ff": ff, "limit": 7.0}
+        raw = {"architecture": "Kazozen", "vocab": vocab, "width": width,
+               "norm": {"eps": 1e-5},
+               "embedding": {"scale": 1.0,
+                             "bigram": {"buckets": 65521, "mul_prev": 37,
+                                        "mul_cur": 19}},
+               "logit_softcap": 30.0,
+               "layers": [
+                   {"type": "attention",
+                    "mixer": mixer(i - 1 if i % 2 else None),
+                    "mlp": dense if i % 2 == 0 else moe}
+                   for i in range(layers)]}
+        mc = model_config_from_dict(raw)
+        mc.name = f"kazozen-{width}x{heads}"
         return mc
     if arch == "momedra":
         # gated attention, latent attention (run twice as a repeated span)

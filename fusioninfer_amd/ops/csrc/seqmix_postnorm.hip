@@ -56,6 +56,23 @@ __global__ __launch_bounds__(256) void pair_embed_kernel(
   __syncthreads();
   const A* e = embed + id * W;
   const A* b = pair_table != nullptr ? pair_table + pair_row * W : nullptr;
+  if (W % 4 == 0) {
+    for (int i = threadIdx.x * 4; i < W; i += 1024) {
+      float x[4], y[4];
+      ldv<A, 4>(e + i, x);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) x[k] *= scale;
+      if (b != nullptr) {
+        ldv<A, 4>(b + i, y);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) x[k] += y[k];
+      }
+      stv<float, 4>(resid + static_cast<int64_t>(t) * W + i, x);
+      if constexpr (!std::is_same<A, float>::value)
+        stv<A, 4>(act + static_cast<int64_t>(t) * W + i, x);
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < W; i += 256) {
     float x = Act<A>::ld(e + i) * scale;
     if (b != nullptr) x += Act<A>::ld(b + i);
@@ -126,8 +143,23 @@ __global__ __launch_bounds__(256) void norm_affine_kernel(
     for (int c = 0; c < NCH; ++c) {
       const int i = (c * 256 + threadIdx.x) * 4;
       if (i < W) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) emit(i + e, v[c][e] * rstd);
+        // 16-byte accesses: weight, bias, stream in and out
+        const float4 w4 = *reinterpret_cast<const float4*>(w + i);
+        const float4 b4 = *reinterpret_cast<const float4*>(b + i);
+        float o4[4] = {v[c][0] * rstd * w4.x + b4.x,
+                       v[c][1] * rstd * w4.y + b4.y,
+                       v[c][2] * rstd * w4.z + b4.z,
+                       v[c][3] * rstd * w4.w + b4.w};
+        if (rr != nullptr) {
+          const float4 r4 = *reinterpret_cast<const float4*>(rr + i);
+          o4[0] += r4.x;
+          o4[1] += r4.y;
+          o4[2] += r4.z;
+          o4[3] += r4.w;
+          *reinterpret_cast<float4*>(rr + i) =
+              float4{o4[0], o4[1], o4[2], o4[3]};
+        }
+        if (orow != nullptr) stv<A, 4>(orow + i, o4);
       }
     }
   } else {
