@@ -173,9 +173,10 @@ def mk(v, device):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("pair", [True, False])
-def test_pair_embedding_and_previous_token_state(device, pair):
+@pytest.mark.parametrize("W", [20, 21])
+def test_pair_embedding_and_previous_token_state(device, pair, W):
     g = torch.Generator().manual_seed(3)
-    V, W, B = 23, 20, 7
+    V, B = 23, 7
     emb = torch.randn(V, W, generator=g)
     tab = torch.randn(B + 1, W, generator=g) if pair else None
     bg = {"buckets": B, "mul_prev": 5, "mul_cur": 3}
